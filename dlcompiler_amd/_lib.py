@@ -1,0 +1,87 @@
+"""ctypes binding of ``libdlblas_hip.so`` (the C ABI declared in ``include/dlblas_hip.h``).
+
+The library is loaded lazily on first use.  If it has not been built the loader raises: there
+is no CPU or eager fallback behind these entry points.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+from pathlib import Path
+
+_PKG_DIR = Path(__file__).resolve().parent
+DEFAULT_LIB_PATH = _PKG_DIR / "lib" / "libdlblas_hip.so"
+
+DLB_OK = 0
+DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
+
+# name -> (restype, argtypes); must list every symbol include/dlblas_hip.h declares
+SIGNATURES = {
+    "dlb_version": (c_int, []),
+    "dlb_status_string": (c_char_p, [c_int]),
+    "dlb_silu_and_mul": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int,
+                                 c_void_p]),
+    "dlb_moe_topk_softmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
+                                         c_int64, c_int, c_void_p]),
+    "dlb_moe_align_ws_bytes": (c_size_t, [c_int64, c_int]),
+    "dlb_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+                                         c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+                                         c_size_t, c_void_p]),
+}
+
+_lib = None
+
+
+class DlblasHipError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+
+def lib_path() -> Path:
+    return Path(os.environ.get("DLBLAS_HIP_LIB", str(DEFAULT_LIB_PATH)))
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once) and attach argument/return types."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not path.exists():
+        raise ImportError(
+            f"{path} not found: build it with `python -m dlcompiler_amd.build` "
+            "(there is no fallback implementation)")
+    lib = ctypes.CDLL(str(path))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != DLB_OK:
+        msg = load().dlb_status_string(status).decode()
+        raise DlblasHipError(f"{what}: {msg} (status {status})")
+
+
+def torch_dtype_code(dtype) -> int:
+    import torch
+
+    table = {torch.bfloat16: DTYPE_BF16, torch.float16: DTYPE_F16, torch.float32: DTYPE_F32}
+    if dtype not in table:
+        raise TypeError(f"unsupported dtype {dtype}")
+    return table[dtype]
+
+
+def current_stream_ptr(device) -> int:
+    import torch
+
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_cuda(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("dlcompiler_amd kernels run on the GPU only; got a CPU tensor")

@@ -1,0 +1,119 @@
+// Shared device/host helpers for the gfx950 kernels of libdlblas_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dlblas_hip.h"
+
+namespace dlb {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+// ---- bf16 / f16 <-> f32 scalar conversions on raw 16-bit patterns -----------------------
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned int b) {
+  return __uint_as_float(b << 16);
+}
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ unsigned int f32_to_bf16_bits(float f) {
+  unsigned int u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ float f16_bits_to_f32(unsigned int b) {
+  _Float16 h = __builtin_bit_cast(_Float16, (unsigned short)b);
+  return (float)h;
+}
+__device__ __forceinline__ unsigned int f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;  // v_cvt_f16_f32: RNE
+  return (unsigned int)__builtin_bit_cast(unsigned short, h);
+}
+
+template <int DT>
+struct Elem;
+template <>
+struct Elem<DLB_DTYPE_BF16> {
+  static __device__ __forceinline__ float lo(unsigned int w) { return __uint_as_float(w << 16); }
+  static __device__ __forceinline__ float hi(unsigned int w) {
+    return __uint_as_float(w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ unsigned int pack(float a, float b) {
+    return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+  }
+  static __device__ __forceinline__ float load1(const void* p, int64_t i) {
+    return bf16_bits_to_f32(((const unsigned short*)p)[i]);
+  }
+  static __device__ __forceinline__ void store1(void* p, int64_t i, float v) {
+    ((unsigned short*)p)[i] = (unsigned short)f32_to_bf16_bits(v);
+  }
+};
+template <>
+struct Elem<DLB_DTYPE_F16> {
+  static __device__ __forceinline__ float lo(unsigned int w) { return f16_bits_to_f32(w & 0xffffu); }
+  static __device__ __forceinline__ float hi(unsigned int w) { return f16_bits_to_f32(w >> 16); }
+  static __device__ __forceinline__ unsigned int pack(float a, float b) {
+    return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+  }
+  static __device__ __forceinline__ float load1(const void* p, int64_t i) {
+    return f16_bits_to_f32(((const unsigned short*)p)[i]);
+  }
+  static __device__ __forceinline__ void store1(void* p, int64_t i, float v) {
+    ((unsigned short*)p)[i] = (unsigned short)f32_to_f16_bits(v);
+  }
+};
+
+// ---- DPP cross-lane moves within a row of 16 lanes ---------------------------------------
+// dpp_ctrl encodings (GCN3+/CDNA): quad_perm = 0x00..0xff, row_mirror = 0x140,
+// row_half_mirror = 0x141.
+constexpr int kDppQuadXor1 = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;  // quad_perm [2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ unsigned int dpp_u32(unsigned int v) {
+  return (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+
+// all-reduce over each aligned group of 16 lanes (a DPP row); every lane gets the result.
+// After the two quad steps all lanes of a quad agree, so the mirror steps (i <-> 7-i,
+// i <-> 15-i) complete a butterfly for any commutative, associative, idempotent-or-not op:
+// each step combines two disjoint halves whose members already hold their half's result.
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f32<kDppQuadXor1>(v));
+  v = fmaxf(v, dpp_f32<kDppQuadXor2>(v));
+  v = fmaxf(v, dpp_f32<kDppRowHalfMirror>(v));
+  v = fmaxf(v, dpp_f32<kDppRowMirror>(v));
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f32<kDppQuadXor1>(v);
+  v += dpp_f32<kDppQuadXor2>(v);
+  v += dpp_f32<kDppRowHalfMirror>(v);
+  v += dpp_f32<kDppRowMirror>(v);
+  return v;
+}
+
+__host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) {
+  return (a + b - 1) / b;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// status of the launch just issued on this thread
+inline int launch_status() { return hipGetLastError() == hipSuccess ? DLB_OK : DLB_ERR_LAUNCH; }
+
+}  // namespace dlb

@@ -1,0 +1,183 @@
+// Expert alignment of MoE routing for gfx950: per-expert counts, expert-sorted flat slot ids
+// padded per expert to a multiple of `block`, and the expert id of each block.
+//
+// The reference derives the same information with a full argsort of the flat id list plus a
+// kernel that rescans that list once per expert
+// (python/dlBLAS/dlblas/kernels/fused_moe.py:238-293, 314-320: exp_start/exp_end are the
+// exclusive/inclusive cumulative sums of the per-expert counts).  Here it is a counting sort:
+//   1. count:  every workgroup histograms its contiguous chunk of the flat id list in LDS and
+//              writes one row of per-chunk counts (plain stores, so the result is reproducible);
+//   2. scan:   one workgroup turns the [chunks, E] table into per-chunk start offsets, pads each
+//              expert's total to `block`, and emits counts, block -> expert ids, the sentinel
+//              pad slots and the padded total;
+//   3. place:  every workgroup re-reads its chunk in order and writes flat index i to
+//              start[chunk][e] + (number of earlier i' in the chunk with the same e), the rank
+//              coming from wave ballots, which makes the sort stable (ascending i per expert).
+// Integer work only; no float or order-dependent atomics, so the output is bit-reproducible.
+#include "common.h"
+
+namespace dlb {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+constexpr int kChunk = 2048;  // flat ids per workgroup
+constexpr int kMaxE = 256;
+
+__host__ __device__ inline int64_t num_chunks(int64_t numel) {
+  return numel > 0 ? (numel + kChunk - 1) / kChunk : 1;
+}
+
+__global__ __launch_bounds__(kThreads) void align_count_kernel(const int32_t* __restrict__ ids,
+                                                               int64_t numel, int E,
+                                                               int32_t* __restrict__ chunk_counts) {
+  __shared__ int32_t hist[kMaxE];
+  for (int e = threadIdx.x; e < E; e += kThreads) hist[e] = 0;
+  __syncthreads();
+  const int64_t begin = (int64_t)blockIdx.x * kChunk;
+  const int64_t end = begin + kChunk < numel ? begin + kChunk : numel;
+  for (int64_t i = begin + threadIdx.x; i < end; i += kThreads) {
+    const int32_t e = ids[i];
+    if (e >= 0 && e < E) atomicAdd(&hist[e], 1);  // integer add: order-insensitive
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kThreads) chunk_counts[(int64_t)blockIdx.x * E + e] = hist[e];
+}
+
+// One workgroup of kMaxE threads; thread e owns expert e.
+__global__ __launch_bounds__(kMaxE) void align_scan_kernel(
+    int32_t* __restrict__ chunk_counts /* in: counts, out: start offsets */, int64_t chunks, int E,
+    int block, int32_t numel, int32_t* __restrict__ sorted_ids, int64_t sorted_cap,
+    int32_t* __restrict__ expert_ids, int64_t expert_ids_cap, int32_t* __restrict__ counts,
+    int32_t* __restrict__ num_post_pad) {
+  __shared__ int32_t padded_s[kMaxE];
+  __shared__ int32_t base_s[kMaxE + 1];
+  const int e = threadIdx.x;
+  int32_t total = 0;
+  if (e < E) {
+    for (int64_t c = 0; c < chunks; ++c) total += chunk_counts[c * E + e];
+  }
+  const int32_t padded = (e < E) ? (int32_t)(ceil_div(total, block) * block) : 0;
+  padded_s[e] = padded;
+  __syncthreads();
+  if (e == 0) {
+    int32_t run = 0;
+    for (int i = 0; i < E; ++i) {
+      base_s[i] = run;
+      run += padded_s[i];
+    }
+    base_s[E] = run;
+    *num_post_pad = run;
+  }
+  __syncthreads();
+  const int32_t total_padded = base_s[E];
+  if (e < E) {
+    const int32_t base = base_s[e];
+    if (counts) counts[e] = total;
+    // chunk start offsets for the placement pass
+    int32_t run = base;
+    for (int64_t c = 0; c < chunks; ++c) {
+      const int32_t n = chunk_counts[c * E + e];
+      chunk_counts[c * E + e] = run;
+      run += n;
+    }
+    // pad slots of this expert
+    for (int32_t p = base + total; p < base + padded; ++p) sorted_ids[p] = numel;
+    // block -> expert
+    for (int32_t b = base / block; b < (base + padded) / block; ++b) expert_ids[b] = e;
+  }
+  // tails beyond the padded total
+  for (int64_t p = (int64_t)total_padded + e; p < sorted_cap; p += kMaxE) sorted_ids[p] = numel;
+  for (int64_t b = (int64_t)total_padded / block + e; b < expert_ids_cap; b += kMaxE)
+    expert_ids[b] = -1;
+}
+
+__global__ __launch_bounds__(kThreads) void align_place_kernel(
+    const int32_t* __restrict__ ids, int64_t numel, int E,
+    const int32_t* __restrict__ chunk_start, int32_t* __restrict__ sorted_ids) {
+  __shared__ int32_t cursor[kMaxE];           // next free slot per expert for this chunk
+  __shared__ int32_t wave_cnt[kWaves][kMaxE];  // per-tile, per-wave counts
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  for (int e = threadIdx.x; e < E; e += kThreads) cursor[e] = chunk_start[(int64_t)blockIdx.x * E + e];
+  for (int i = threadIdx.x; i < kWaves * kMaxE; i += kThreads) (&wave_cnt[0][0])[i] = 0;
+  __syncthreads();
+
+  const int64_t begin = (int64_t)blockIdx.x * kChunk;
+  const int64_t end = begin + kChunk < numel ? begin + kChunk : numel;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int64_t tile = begin; tile < end; tile += kThreads) {  // uniform trip count
+    const int64_t i = tile + threadIdx.x;
+    int32_t e = -1;
+    if (i < end) {
+      e = ids[i];
+      if (e < 0 || e >= E) e = -1;
+    }
+    // lanes of this wave holding the same expert: intersect ballots over the 9 key bits
+    // (bit 8 separates the dropped entries, e = -1 -> key 0x1ff).
+    const uint32_t key = (uint32_t)e & 0x1ffu;
+    uint64_t peers = ~0ull;
+#pragma unroll
+    for (int b = 0; b < 9; ++b) {
+      const bool bit = (key >> b) & 1u;
+      const uint64_t m = __ballot(bit);
+      peers &= bit ? m : ~m;
+    }
+    const int rank_in_wave = __popcll(peers & lt_mask);
+    const int peer_count = __popcll(peers);
+    if (e >= 0 && rank_in_wave == 0) wave_cnt[wave][e] = peer_count;
+    __syncthreads();
+    if (e >= 0) {
+      int32_t pos = cursor[e] + rank_in_wave;
+      for (int w = 0; w < wave; ++w) pos += wave_cnt[w][e];
+      sorted_ids[pos] = (int32_t)i;
+    }
+    __syncthreads();
+    for (int x = threadIdx.x; x < E; x += kThreads) {
+      int32_t add = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        add += wave_cnt[w][x];
+        wave_cnt[w][x] = 0;
+      }
+      cursor[x] += add;
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace
+}  // namespace dlb
+
+extern "C" size_t dlb_moe_align_ws_bytes(int64_t numel, int E) {
+  if (numel < 0 || E < 1) return 0;
+  return (size_t)dlb::num_chunks(numel) * (size_t)E * sizeof(int32_t);
+}
+
+extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int block,
+                                        int32_t* sorted_ids, int64_t sorted_cap,
+                                        int32_t* expert_ids, int64_t expert_ids_cap,
+                                        int32_t* counts, int32_t* num_post_pad, void* ws,
+                                        size_t ws_bytes, void* stream) {
+  using namespace dlb;
+  if (numel < 0 || E < 1 || block < 1) return DLB_ERR_BAD_ARG;
+  if (E > kMaxE) return DLB_ERR_UNSUPPORTED;
+  if (numel + (int64_t)E * block >= (int64_t)0x7fffffff) return DLB_ERR_UNSUPPORTED;
+  if (!sorted_ids || !expert_ids || !num_post_pad || (numel > 0 && !topk_ids))
+    return DLB_ERR_BAD_ARG;
+  if (sorted_cap < numel + (int64_t)E * (block - 1)) return DLB_ERR_BAD_ARG;
+  if (expert_ids_cap < ceil_div(sorted_cap, block)) return DLB_ERR_BAD_ARG;
+  if (!ws || ws_bytes < dlb_moe_align_ws_bytes(numel, E)) return DLB_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t chunks = num_chunks(numel);
+  int32_t* chunk_counts = (int32_t*)ws;
+  hipLaunchKernelGGL(align_count_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
+                     numel, E, chunk_counts);
+  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kMaxE), 0, s, chunk_counts, chunks, E, block,
+                     (int32_t)numel, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, counts,
+                     num_post_pad);
+  if (numel > 0)
+    hipLaunchKernelGGL(align_place_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
+                       numel, E, chunk_counts, sorted_ids);
+  return launch_status();
+}

@@ -1,0 +1,157 @@
+// MoE router for gfx950: softmax over experts, top-k selection, optional renormalisation.
+//
+// Semantics follow the router the reference's fused_moe is fed with
+// (python/dlBLAS/tests/kernels/test_fused_moe.py:213-216: softmax in fp32, then top-k;
+// python/dlBLAS/dlblas/kernels/fused_moe.py:322-323: weights / weights.sum(-1)), with the two
+// points the reference leaves open fixed here: selection runs on the logits (the softmax is
+// monotone, so this is the same order without depending on exp rounding) and equal logits
+// resolve to the lowest expert index.  The fused softmax + K x argmax structure is that of
+// python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:24-60, minus its [K, S, E] int64
+// one-hot masks: indices are written directly.
+//
+// Mapping: a token is owned by one DPP row (16 lanes); every lane holds VPL consecutive
+// experts (VPL = 4 covers E <= 64 with one 128-bit load per lane), so a wave processes four
+// tokens and every reduction (max, sum, K argmax rounds) is four DPP steps with no LDS.
+#include "common.h"
+
+namespace dlb {
+namespace {
+
+// order-preserving map float -> uint32 (larger float <=> larger key); -0.0 < +0.0 there, so
+// canonicalise zeros first to keep "equal logits -> lowest index".
+__device__ __forceinline__ uint32_t orderable(float f) {
+  f = (f == 0.0f) ? 0.0f : f;
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// max of (key, tag) pairs over a DPP row, lexicographic on (key, tag).
+template <int CTRL>
+__device__ __forceinline__ void row_step_max(uint32_t& key, uint32_t& tag) {
+  const uint32_t ok = dpp_u32<CTRL>(key);
+  const uint32_t ot = dpp_u32<CTRL>(tag);
+  const bool take = (ok > key) || (ok == key && ot > tag);
+  key = take ? ok : key;
+  tag = take ? ot : tag;
+}
+
+template <int VPL>
+__global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
+    const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
+    int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok) {
+  const int lane16 = threadIdx.x & 15;
+  const int64_t token = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  // every lane of a row takes the same branch; DPP rows never straddle tokens
+  const bool live = token < T;
+  const float NEG_INF = -__builtin_inff();
+
+  float v[VPL];
+  const int e0 = lane16 * VPL;
+  if (live && vec_ok) {
+    const f32x4* p = reinterpret_cast<const f32x4*>(logits + token * ld + e0);
+#pragma unroll
+    for (int q = 0; q < VPL / 4; ++q) {
+      const f32x4 t = p[q];
+      v[4 * q + 0] = t[0];
+      v[4 * q + 1] = t[1];
+      v[4 * q + 2] = t[2];
+      v[4 * q + 3] = t[3];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      v[j] = (live && e0 + j < E) ? logits[token * ld + e0 + j] : NEG_INF;
+  }
+
+  // softmax statistics: p_e = exp(l_e - max) / sum
+  float mx = v[0];
+#pragma unroll
+  for (int j = 1; j < VPL; ++j) mx = fmaxf(mx, v[j]);
+  mx = row16_max(mx);
+  float ex[VPL];
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    ex[j] = expf(v[j] - mx);  // exp(-inf) = 0 for the padding experts
+    sum += ex[j];
+  }
+  sum = row16_sum(sum);
+
+  // K rounds of arg-max over (orderable(logit), 256 - index): ties -> lowest index.
+  // tag 0 means "no candidate"; real candidates carry tag = 256 - index >= 1.
+  uint32_t key[VPL];
+  uint32_t alive = 0u;
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    key[j] = orderable(v[j]);
+    alive |= (e0 + j < E) ? (1u << j) : 0u;
+  }
+
+  float my_w = 0.0f;  // lane r keeps the r-th selected probability
+  int32_t my_id = 0;
+  float wsum = 0.0f;
+  for (int r = 0; r < K; ++r) {
+    uint32_t bk = 0u, bt = 0u;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      // strict '>' keeps the lowest index among equal keys inside the lane (j ascending)
+      if (((alive >> j) & 1u) && (bt == 0u || key[j] > bk)) {
+        bk = key[j];
+        bt = (uint32_t)(256 - (e0 + j));
+      }
+    }
+    row_step_max<kDppQuadXor1>(bk, bt);
+    row_step_max<kDppQuadXor2>(bk, bt);
+    row_step_max<kDppRowHalfMirror>(bk, bt);
+    row_step_max<kDppRowMirror>(bk, bt);
+    const int sel = 256 - (int)bt;  // winning expert, identical on all 16 lanes
+    float p = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      if (e0 + j == sel) {
+        p = ex[j] / sum;
+        alive &= ~(1u << j);
+      }
+    }
+    // only the owner lane holds a non-zero p; x + 0 + ... + 0 == x, so the row sum is a
+    // bit-exact broadcast.
+    p = row16_sum(p);
+    wsum += p;
+    if (lane16 == r) {
+      my_w = p;
+      my_id = sel;
+    }
+  }
+  if (live && lane16 < K) {
+    const float w = renorm ? my_w / wsum : my_w;
+    weights[token * K + lane16] = w;
+    ids[token * K + lane16] = my_id;
+  }
+}
+
+}  // namespace
+}  // namespace dlb
+
+extern "C" int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids,
+                                        int64_t T, int E, int K, int64_t ld_logits,
+                                        int renormalize, void* stream) {
+  using namespace dlb;
+  if (T < 0 || E < 1 || K < 1 || K > E || ld_logits < E) return DLB_ERR_BAD_ARG;
+  if (K > 16 || E > 256) return DLB_ERR_UNSUPPORTED;
+  if (T == 0) return DLB_OK;
+  if (!logits || !weights || !ids) return DLB_ERR_BAD_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((uint32_t)ceil_div(T, 16)), block(256);
+  const bool a16 = aligned16(logits) && (ld_logits % 4 == 0);
+  if (E <= 64) {
+    hipLaunchKernelGGL(moe_topk_softmax_kernel<4>, grid, block, 0, s, logits, weights, ids, T, E,
+                       K, ld_logits, renormalize, (int)(a16 && E == 64));
+  } else if (E <= 128) {
+    hipLaunchKernelGGL(moe_topk_softmax_kernel<8>, grid, block, 0, s, logits, weights, ids, T, E,
+                       K, ld_logits, renormalize, (int)(a16 && E == 128));
+  } else {
+    hipLaunchKernelGGL(moe_topk_softmax_kernel<16>, grid, block, 0, s, logits, weights, ids, T, E,
+                       K, ld_logits, renormalize, (int)(a16 && E == 256));
+  }
+  return launch_status();
+}

@@ -1,0 +1,84 @@
+"""MoE routing operators: router softmax/top-k and expert block alignment.
+
+The reference has no single entry point for these: the router is done by the caller in torch
+(python/dlBLAS/tests/kernels/test_fused_moe.py:213-216, renormalise at
+python/dlBLAS/dlblas/kernels/fused_moe.py:322-323) and the sort/ranges by ``fused_moe`` itself
+(fused_moe.py:267-293, 314-320).  The names below are this package's own.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+
+def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True):
+    """softmax(logits, fp32) -> top-k -> (optionally) weights / weights.sum(-1).
+
+    Returns ``(weights fp32 [T, k], ids int32 [T, k])`` ordered by descending logit, equal
+    logits resolving to the lowest expert index.
+    """
+    assert logits.dim() == 2
+    _lib.require_cuda(logits)
+    T, E = logits.shape
+    if not 1 <= k <= E:
+        raise ValueError(f"need 1 <= k <= num_experts, got k={k}, E={E}")
+    if logits.dtype != torch.float32:
+        logits = logits.float()
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    weights = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    if T > 0:
+        lib = _lib.load()
+        with torch.cuda.device(logits.device):
+            st = lib.dlb_moe_topk_softmax_f32(logits.data_ptr(), weights.data_ptr(),
+                                              ids.data_ptr(), T, E, k,
+                                              logits.stride(0) if T > 1 else E,
+                                              int(bool(renormalize)),
+                                              _lib.current_stream_ptr(logits.device))
+        _lib.check(st, "dlb_moe_topk_softmax_f32")
+    return weights, ids
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int,
+                         return_counts: bool = False):
+    """Group the flat routing slots ``i = token * k + j`` by expert, padded to ``block_size``.
+
+    Returns ``(sorted_token_ids, expert_ids, num_tokens_post_padded[, counts])``, all int32:
+
+    * ``sorted_token_ids`` has length ``numel + num_experts * (block_size - 1)``; expert
+      segments in expert order, each a multiple of ``block_size`` long with that expert's flat
+      indices ascending; every other slot holds the sentinel ``numel``;
+    * ``expert_ids[b]`` is the expert of block ``b`` (``-1`` past the padded total);
+    * ``num_tokens_post_padded`` is a 1-element tensor; ``counts[e]`` the tokens of expert e.
+
+    Ids outside ``[0, num_experts)`` are dropped (experts held by another shard).
+    """
+    _lib.require_cuda(topk_ids)
+    if block_size < 1 or num_experts < 1:
+        raise ValueError("block_size and num_experts must be positive")
+    ids = topk_ids.reshape(-1)
+    if ids.dtype != torch.int32:
+        ids = ids.to(torch.int32)
+    ids = ids.contiguous()
+    numel = ids.numel()
+    dev = ids.device
+    cap = numel + num_experts * (block_size - 1)
+    nblk = max(1, -(-cap // block_size))
+    sorted_ids = torch.empty((cap,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((nblk,), dtype=torch.int32, device=dev)
+    num_post = torch.empty((1,), dtype=torch.int32, device=dev)
+    counts = torch.empty((num_experts,), dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    ws_bytes = lib.dlb_moe_align_ws_bytes(numel, num_experts)
+    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.dlb_moe_align_block_size(ids.data_ptr(), numel, num_experts, block_size,
+                                          sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk,
+                                          counts.data_ptr(), num_post.data_ptr(), ws.data_ptr(),
+                                          ws.numel(), _lib.current_stream_ptr(dev))
+    _lib.check(st, "dlb_moe_align_block_size")
+    if return_counts:
+        return sorted_ids, expert_ids, num_post, counts
+    return sorted_ids, expert_ids, num_post

@@ -1,0 +1,96 @@
+/*
+ * dlblas_hip.h -- C ABI of libdlblas_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * dlBLAS LLM-inference operator set.
+ *
+ * The reference library (DLCompiler's dlBLAS) has no FFI boundary: its Python host wrappers
+ * launch Triton kernels.  Each entry point below replaces one such "host wrapper -> Triton
+ * launch" pair; the reference location is cited per function as
+ * python/dlBLAS/dlblas/kernels/<file>:<lines>.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers to DEVICE memory, sizes and strides in ELEMENTS unless stated otherwise;
+ *   - the library never allocates or frees: outputs and workspaces are caller-owned;
+ *   - `stream` is a hipStream_t passed as void*; every call is asynchronous on it, re-entrant,
+ *     and holds no mutable global state;
+ *   - return value: DLB_OK (0) or a negative DLB_ERR_* code; nothing is launched on error.
+ */
+#ifndef DLBLAS_HIP_H_
+#define DLBLAS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DLB_OK 0
+#define DLB_ERR_BAD_ARG (-1)     /* null pointer, negative size, inconsistent shapes        */
+#define DLB_ERR_UNSUPPORTED (-2) /* legal request the kernels do not cover (shape/dtype)    */
+#define DLB_ERR_LAUNCH (-3)      /* hipGetLastError() != hipSuccess after the launch        */
+#define DLB_ERR_WORKSPACE (-4)   /* workspace pointer null or too small                     */
+
+/* element types of activations */
+#define DLB_DTYPE_BF16 0
+#define DLB_DTYPE_F16 1
+#define DLB_DTYPE_F32 2
+
+/* ABI version: bumped whenever a signature below changes. */
+int dlb_version(void);
+/* static string for a status code (never NULL). */
+const char* dlb_status_string(int status);
+
+/* ------------------------------------------------------------------------------------------
+ * silu_and_mul: out[m, j] = silu(x[m, j]) * x[m, N + j], math in fp32, one rounding to dtype.
+ * Replaces silu_and_mul + _silu_and_mul[_no_align]_kernel, kernels/activation.py:17-130.
+ *   x   [M, 2N] row stride ld_x (elements), unit column stride
+ *   out [M, N]  row stride ld_out
+ * Any M >= 0, N >= 0; a 128-bit vector path is taken when N % 8 == 0 (bf16/f16) or N % 4 == 0
+ * (f32) and pointers/strides are 16-byte aligned, otherwise an element-wise path.
+ * ---------------------------------------------------------------------------------------- */
+int dlb_silu_and_mul(const void* x, void* out, int64_t M, int64_t N, int64_t ld_x,
+                     int64_t ld_out, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * moe_topk_softmax: router softmax over experts + top-k (+ renormalise).
+ * Replaces the router the reference leaves to the caller in torch
+ * (tests/kernels/test_fused_moe.py:213-216: softmax(fp32) then torch.topk; renormalise
+ * kernels/fused_moe.py:322-323) and the fused softmax+argmax of
+ * kernels/topk_gating_fwd_part1.py:24-60.
+ *   logits  fp32 [T, E], row stride ld_logits
+ *   weights fp32 [T, K] (contiguous) ; ids int32 [T, K] (contiguous)
+ * Selection is on the logits, descending, ties to the LOWEST expert index; weights are
+ * p = exp(l - max) / sum(exp(l - max)) of the selected experts, divided by their sum when
+ * renormalize != 0.  1 <= K <= 16, K <= E <= 256.
+ * ---------------------------------------------------------------------------------------- */
+int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids, int64_t T,
+                             int E, int K, int64_t ld_logits, int renormalize, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * moe_align_block_size: per-expert counts, expert-sorted flat slot ids padded per expert to a
+ * multiple of `block`, and the expert of every block.
+ * Replaces the routing bookkeeping of fused_moe: argsort + get_start_end/_start_end_kernel,
+ * kernels/fused_moe.py:238-293,314-320 (the pad-to-block layout itself has no reference
+ * counterpart).
+ *   topk_ids    int32 [numel]  (flat index i = token * K + j); ids outside [0, E) are dropped
+ *   sorted_ids  int32 [sorted_cap], sorted_cap >= numel + E * (block - 1):
+ *               expert segments in expert order, each a multiple of `block` long, holding the
+ *               flat indices of that expert ASCENDING, then pad slots; every slot that is not
+ *               a real entry (pads and the tail up to sorted_cap) holds the sentinel `numel`
+ *   expert_ids  int32 [expert_ids_cap], expert_ids_cap >= ceil(sorted_cap / block):
+ *               expert of block b for b < num_post_pad / block, -1 after
+ *   counts      int32 [E] tokens per expert (may be NULL)
+ *   num_post_pad int32 [1] total padded length
+ *   ws          device scratch of dlb_moe_align_ws_bytes(numel, E) bytes
+ * 1 <= E <= 256, block >= 1, numel < 2^31 - E * block.
+ * ---------------------------------------------------------------------------------------- */
+size_t dlb_moe_align_ws_bytes(int64_t numel, int E);
+int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int block,
+                             int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids,
+                             int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
+                             void* ws, size_t ws_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DLBLAS_HIP_H_ */

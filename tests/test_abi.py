@@ -1,0 +1,62 @@
+"""The C-ABI library loads and exports exactly what include/dlblas_hip.h declares (no GPU)."""
+import re
+from pathlib import Path
+
+import pytest
+
+from dlcompiler_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "dlblas_hip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dlb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_something():
+    assert "dlb_silu_and_mul" in _declared_symbols()
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == declared, "ctypes table and header disagree"
+
+
+def test_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.dlb_version() >= 1
+    assert lib.dlb_status_string(0) == b"ok"
+    for code in (-1, -2, -3, -4, -99):
+        assert lib.dlb_status_string(code)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setenv("DLBLAS_HIP_LIB", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_lib, "_lib", None)
+    with pytest.raises(ImportError):
+        _lib.load()
+
+
+def test_cpu_tensor_is_rejected():
+    import torch
+
+    from dlcompiler_amd import silu_and_mul
+
+    with pytest.raises(ValueError):
+        silu_and_mul(torch.zeros(2, 8, dtype=torch.bfloat16))
+
+
+def test_argument_validation_needs_no_gpu():
+    # status codes for bad arguments are produced on the host before any launch
+    lib = _lib.load()
+    assert lib.dlb_silu_and_mul(None, None, -1, 8, 16, 8, 0, None) == -1
+    assert lib.dlb_silu_and_mul(None, None, 4, 8, 8, 8, 0, None) == -1  # ld_x < 2N
+    assert lib.dlb_silu_and_mul(None, None, 0, 8, 16, 8, 0, None) == 0  # empty is fine
+    assert lib.dlb_moe_topk_softmax_f32(None, None, None, 4, 64, 65, 64, 1, None) == -1
+    assert lib.dlb_moe_topk_softmax_f32(None, None, None, 4, 512, 2, 512, 1, None) == -2
+    assert lib.dlb_moe_align_ws_bytes(98304, 64) > 0

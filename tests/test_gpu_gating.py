@@ -1,0 +1,122 @@
+"""GPU parity: router softmax/top-k and expert alignment vs the CPU oracle (C ABI path)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_gating as og
+from test_oracle_gating import check_align_invariants
+
+pytestmark = pytest.mark.gpu
+
+
+def _topk(logits_cpu, k, dev, renorm=True):
+    from dlcompiler_amd.kernels.moe_gating import moe_topk_softmax
+
+    w, ids = moe_topk_softmax(logits_cpu.to(dev), k, renormalize=renorm)
+    assert w.dtype == torch.float32 and ids.dtype == torch.int32
+    return w.cpu(), ids.cpu()
+
+
+@pytest.mark.parametrize("T,E,k", [(16384, 64, 6), (128, 4, 2), (4096, 64, 8), (1, 64, 6),
+                                   (77, 8, 2), (333, 60, 6), (100, 128, 8), (50, 160, 6),
+                                   (19, 256, 16), (5, 3, 3)])
+@pytest.mark.parametrize("renorm", [True, False])
+def test_topk_softmax_parity(dev, T, E, k, renorm):
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn((T, E), generator=g)
+    w, ids = _topk(logits, k, dev, renorm)
+    rw, rids = og.topk_softmax(logits, k, renormalize=renorm)
+    assert torch.equal(ids, rids)                               # bit-exact indices
+    torch.testing.assert_close(w, rw, rtol=1e-6, atol=0)        # north-star: 1e-6 relative
+
+
+def test_topk_ties_resolve_to_lowest_index(dev):
+    logits = torch.zeros((40, 64))
+    logits[1, 10:20] = 2.0
+    logits[2] = torch.arange(64).float().flip(0)
+    logits[3, ::2] = 1.0
+    logits[4, 5] = -0.0
+    g = torch.Generator().manual_seed(9)
+    logits[8:] = torch.randint(-2, 3, (32, 64), generator=g).float()   # many ties
+    w, ids = _topk(logits, 6, dev)
+    rw, rids = og.topk_softmax(logits, 6)
+    assert ids[0].tolist() == [0, 1, 2, 3, 4, 5]
+    assert ids[1].tolist() == [10, 11, 12, 13, 14, 15]
+    assert ids[3].tolist() == [0, 2, 4, 6, 8, 10]
+    assert ids[4].tolist() == [0, 1, 2, 3, 4, 5]
+    assert torch.equal(ids, rids)
+    torch.testing.assert_close(w, rw, rtol=1e-6, atol=0)
+
+
+def test_topk_strided_and_extreme_logits(dev):
+    from dlcompiler_amd.kernels.moe_gating import moe_topk_softmax
+
+    g = torch.Generator().manual_seed(4)
+    wide = torch.randn((64, 200), generator=g) * 30.0           # exp would overflow unshifted
+    view = wide[:, 3:67]
+    w, ids = moe_topk_softmax(wide.to(dev)[:, 3:67], 6)
+    rw, rids = og.topk_softmax(view.contiguous(), 6)
+    assert torch.equal(ids.cpu(), rids)
+    torch.testing.assert_close(w.cpu(), rw, rtol=1e-6, atol=1e-30)
+
+
+def _align(ids_cpu, block, E, dev):
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size
+
+    out = moe_align_block_size(ids_cpu.to(dev), block, E, return_counts=True)
+    return [t.cpu() for t in out]
+
+
+@pytest.mark.parametrize("T,k,E,block", [(16384, 6, 64, 64), (4096, 6, 64, 64), (128, 2, 4, 16),
+                                         (1, 6, 64, 64), (7, 3, 5, 1), (1000, 8, 256, 128),
+                                         (3000, 4, 60, 32), (2048, 1, 2, 64), (513, 2, 160, 8)])
+def test_align_bit_exact(dev, T, k, E, block):
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn((T, E), generator=g)
+    _, ids = og.topk_softmax(logits, k)
+    s, e, tot, cnt = _align(ids, block, E, dev)
+    rs, re_, rtot, rcnt = og.align_block_size(ids, block, E)
+    assert torch.equal(cnt, rcnt) and torch.equal(tot, rtot)
+    assert torch.equal(e, re_)
+    assert torch.equal(s, rs)
+    check_align_invariants(ids.flatten().numpy(), block, E, s, e, tot.item(), cnt)
+    # reference view of the same data: exp_start/exp_end (fused_moe.py:271-275)
+    start, end = og.start_end(ids, E)
+    assert torch.equal(end - start, cnt.long())
+
+
+def test_align_empty_skewed_and_dropped(dev):
+    s, e, tot, cnt = _align(torch.zeros((0, 6), dtype=torch.int32), 64, 64, dev)
+    assert tot.item() == 0 and cnt.sum() == 0 and (s == 0).all() and (e == -1).all()
+    # every slot on one expert; and a list with ids owned by another shard
+    for ids in [torch.full((5000, 2), 3, dtype=torch.int32),
+                torch.tensor([[0, 70], [-1, 1], [1, 64], [63, 0]], dtype=torch.int32)]:
+        out = _align(ids, 64, 64, dev)
+        ref = og.align_block_size(ids, 64, 64)
+        for a, b in zip(out, ref):
+            assert torch.equal(a, b)
+
+
+def test_align_is_deterministic(dev):
+    g = torch.Generator().manual_seed(11)
+    ids = torch.randint(0, 64, (16384, 6), generator=g, dtype=torch.int32)
+    first = _align(ids, 64, 64, dev)
+    for _ in range(3):
+        again = _align(ids, 64, 64, dev)
+        assert all(torch.equal(a, b) for a, b in zip(first, again))
+
+
+def test_end_to_end_config2(dev):
+    # BASELINE config 2: logits fp32 [16384, 64] ~ N(0,1) seed 1, k = 6, block 64
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size, moe_topk_softmax
+
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn((16384, 64), generator=g)
+    w, ids = moe_topk_softmax(logits.to(dev), 6)
+    s, e, tot = moe_align_block_size(ids, 64, 64)
+    rw, rids = og.topk_softmax(logits, 6)
+    rs, re_, rtot, _ = og.align_block_size(rids, 64, 64)
+    assert torch.equal(ids.cpu(), rids) and torch.equal(s.cpu(), rs)
+    assert torch.equal(e.cpu(), re_) and tot.item() == rtot.item()
+    torch.testing.assert_close(w.cpu(), rw, rtol=1e-6, atol=0)
+    np.testing.assert_allclose(w.cpu().sum(-1).numpy(), 1.0, atol=3e-7)
