@@ -28,6 +28,9 @@ SIGNATURES = {
     "dlb_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                          c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                          c_size_t, c_void_p]),
+    "dlb_paged_decode_ws_bytes": (c_size_t, [c_int] * 6),
+    "dlb_paged_decode_attn": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_int64] * 11
+                              + [c_float, c_int, c_void_p, c_size_t, c_void_p]),
 }
 
 _lib = None

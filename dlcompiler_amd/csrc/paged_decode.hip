@@ -1,0 +1,393 @@
+// Paged decode attention for gfx950: one query token per sequence, KV cache in fixed-size
+// pages addressed through a block table, grouped-query heads.
+//
+// Replaces the decode branch of paged_attention_fwd
+// (python/dlBLAS/dlblas/kernels/paged_attention.py:604-671): _fwd_grouped_split_kernel
+// (:45-234) and _reduce_split_kernel (:238-285).  Same mathematics -- per (sequence, kv head)
+// the query heads of the group are batched against the head's K/V stream, online softmax in
+// fp32, P rounded to the cache dtype before P.V, split-KV partials (O, m, l) combined by a
+// second kernel -- with a different decomposition:
+//   * a work item is (sequence, kv head, KV chunk of `keys_per_split` tokens) instead of a
+//     fixed four-way split, so items are equally long whatever the context length;
+//   * one wavefront per item.  S^T = K.Q^T runs on 16x16x32 MFMA with the K rows loaded
+//     straight from HBM into the A-operand layout (d is contiguous in memory and in the
+//     operand), so K never touches LDS;
+//   * V needs the key index contiguous per lane, so its tile is transposed on the way into
+//     LDS (4 keys x 8 dims per lane, v_perm + ds_write_b64) and read back as 128-bit operands;
+//     the key order inside each 32-key MFMA step is permuted so that the softmax output
+//     registers ARE the B operand of O^T = V^T.P^T: P never moves between lanes.
+// The kernel is an HBM stream (4 FLOP/byte at GQA 4:1); everything else is sized to keep
+// tens of KB of loads in flight per CU.
+#include "common.h"
+
+namespace dlb {
+namespace {
+
+struct DecodeParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  const int32_t* block_table;
+  const int32_t* kv_len;
+  float* ws_o;   // [B, Hq, nsplit_max, D]
+  float* ws_ml;  // [B, Hq, nsplit_max, 2]
+  int64_t q_sb, q_sh;
+  int64_t k_sp, k_st, k_sh;
+  int64_t v_sp, v_st, v_sh;
+  int64_t o_sb, o_sh;
+  int64_t bt_stride;
+  int B, Hq, Hkv, group, hchunks;
+  int page, page_shift;  // page_shift < 0: page is not a power of two
+  int max_blocks;
+  int keys_per_split, nsplit_max;
+  float scale_log2e;
+};
+
+template <int DT>
+struct Mma16;
+template <>
+struct Mma16<DLB_DTYPE_BF16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned int pack2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+    f2 f = {a, b};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, b2));
+  }
+};
+template <>
+struct Mma16<DLB_DTYPE_F16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ unsigned int pack2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    f2 f = {a, b};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, h2));
+  }
+};
+
+constexpr int kTile = 64;          // keys per iteration
+constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
+
+template <int DT, int D>
+__global__ __launch_bounds__(64) void paged_decode_split_kernel(const DecodeParams p) {
+  constexpr int KS = D / 32;   // MFMA k-steps over the head dim
+  constexpr int MT = D / 16;   // 16-row tiles of O^T
+  constexpr int VIT = D / 32;  // V staging iterations (64 lanes x 4 keys x 8 dims each)
+  constexpr int DG = D / 8;    // 8-dim groups per key row
+
+  const int split = blockIdx.x;
+  const int kvh = blockIdx.y / p.hchunks;
+  const int hchunk = blockIdx.y - kvh * p.hchunks;
+  const int b = blockIdx.z;
+  const int ctx = p.kv_len[b];
+  const int k_begin = split * p.keys_per_split;
+  if (k_begin >= ctx) return;  // uniform for the wave; also covers ctx <= 0
+  const int k_end = min(ctx, k_begin + p.keys_per_split);
+
+  const int lane = threadIdx.x;
+  const int g = lane >> 4;  // lane group 0..3
+  const int c = lane & 15;  // column (query head) / row (key) inside a 16-tile
+
+  __shared__ __attribute__((aligned(16))) unsigned char vt[D * kVtRowBytes];
+
+  const unsigned short* qb = (const unsigned short*)p.q;
+  const unsigned short* kb = (const unsigned short*)p.k;
+  const unsigned short* vb = (const unsigned short*)p.v;
+  const int32_t* bt = p.block_table + (int64_t)b * p.bt_stride;
+
+  // Q^T as the B operand: lane (n = query head c, k = dims 32*ks + 8g .. +8)
+  const int hq_local = hchunk * 16 + c;
+  const bool head_ok = hq_local < p.group;
+  const int head = kvh * p.group + hq_local;
+  u32x4 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    qf[ks] = u32x4{0u, 0u, 0u, 0u};
+    if (head_ok)
+      qf[ks] = *(const u32x4*)(qb + (int64_t)b * p.q_sb + (int64_t)head * p.q_sh + 32 * ks + 8 * g);
+  }
+
+  f32x4 o[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) o[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -__builtin_inff();
+  float l_run = 0.0f;  // per-lane partial of the softmax denominator
+
+  auto page_of = [&](int key, int& in_page) -> int64_t {
+    int pi;
+    if (p.page_shift >= 0) {
+      pi = key >> p.page_shift;
+      in_page = key & (p.page - 1);
+    } else {
+      pi = key / p.page;
+      in_page = key - pi * p.page;
+    }
+    return (int64_t)bt[pi];
+  };
+
+  for (int t0 = k_begin; t0 < k_end; t0 += kTile) {
+    // ---- K tile: 4 sub-tiles of 16 keys, straight into A-operand registers ----
+    u32x4 kf[4][KS];
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      const int key = min(t0 + 16 * sub + c, ctx - 1);  // clamp: never read past the context
+      int in_page;
+      const int64_t pg = page_of(key, in_page);
+      const unsigned short* kp = kb + pg * p.k_sp + (int64_t)in_page * p.k_st + (int64_t)kvh * p.k_sh;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kf[sub][ks] = *(const u32x4*)(kp + 32 * ks + 8 * g);
+    }
+    // ---- V tile: each lane takes 4 consecutive keys x 8 dims per iteration ----
+    u32x4 vr[VIT][4];
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
+      const int u = it * 64 + lane;
+      const int dg = u % DG, kg = u / DG;
+      const int key0 = min(t0 + 4 * kg, ctx - 1);
+      int in_page;
+      const int64_t pg = page_of(key0, in_page);
+      const unsigned short* vp = vb + pg * p.v_sp + (int64_t)kvh * p.v_sh + 8 * dg;
+      // the 4 keys share a page (page % 16 == 0); clamp each inside the context
+      const int room = ctx - 1 - key0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rr = min(r, room);
+        vr[it][r] = *(const u32x4*)(vp + (int64_t)(in_page + rr) * p.v_st);
+      }
+    }
+
+    // ---- S^T = K . Q^T (rows = keys, cols = query heads) ----
+    f32x4 s[4];
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      s[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s[sub] = Mma16<DT>::run(kf[sub][ks], qf[ks], s[sub]);
+    }
+
+    // ---- V^T into LDS: Vt[d][pos], pos = 32*s + 8*g' + 4*a + r for key 32*s + 16*a + 4*g' + r
+    __syncthreads();  // previous tile's operand reads are done
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
+      const int u = it * 64 + lane;
+      const int dg = u % DG, kg = u / DG;
+      const int unit = 4 * (kg >> 3) + (kg & 3);  // 16-byte unit inside the row
+      const int half = (kg >> 2) & 1;             // 8-byte half inside the unit
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const unsigned int lo01 = __builtin_amdgcn_perm(vr[it][1][w], vr[it][0][w], 0x05040100u);
+        const unsigned int lo23 = __builtin_amdgcn_perm(vr[it][3][w], vr[it][2][w], 0x05040100u);
+        const unsigned int hi01 = __builtin_amdgcn_perm(vr[it][1][w], vr[it][0][w], 0x07060302u);
+        const unsigned int hi23 = __builtin_amdgcn_perm(vr[it][3][w], vr[it][2][w], 0x07060302u);
+        const int d0 = 8 * dg + 2 * w;
+        const int sw = ((d0 >> 4) & 3) << 1;  // same for d0 and d0 + 1
+        unsigned char* row = vt + d0 * kVtRowBytes + ((unit ^ sw) << 4) + (half << 3);
+        *(u32x2*)(row) = u32x2{lo01, lo23};
+        *(u32x2*)(row + kVtRowBytes) = u32x2{hi01, hi23};
+      }
+    }
+
+    // ---- online softmax over this tile (log2 domain) ----
+    float mloc = -__builtin_inff();
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = t0 + 16 * sub + 4 * g + i;
+        const float x = (key < k_end) ? s[sub][i] * p.scale_log2e : -__builtin_inff();
+        s[sub][i] = x;
+        mloc = fmaxf(mloc, x);
+      }
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    const float m_new = fmaxf(m_run, mloc);  // finite: key t0 is always valid
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    float psum = 0.0f;
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e = __builtin_amdgcn_exp2f(s[sub][i] - m_new);
+        s[sub][i] = e;
+        psum += e;
+      }
+    }
+    l_run = l_run * alpha + psum;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+
+    // P^T as B operand of step st: slots 0..3 <- sub-tile 2*st, slots 4..7 <- sub-tile 2*st+1
+    u32x4 pf[2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      pf[st][0] = Mma16<DT>::pack2(s[2 * st][0], s[2 * st][1]);
+      pf[st][1] = Mma16<DT>::pack2(s[2 * st][2], s[2 * st][3]);
+      pf[st][2] = Mma16<DT>::pack2(s[2 * st + 1][0], s[2 * st + 1][1]);
+      pf[st][3] = Mma16<DT>::pack2(s[2 * st + 1][2], s[2 * st + 1][3]);
+    }
+
+    __syncthreads();  // V^T tile visible
+    // ---- O^T += V^T . P^T ----
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int d = 16 * mt + c;
+      const int sw = (mt & 3) << 1;
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const u32x4 a = *(const u32x4*)(vt + d * kVtRowBytes + (((4 * st + g) ^ sw) << 4));
+        o[mt] = Mma16<DT>::run(a, pf[st], o[mt]);
+      }
+    }
+  }
+
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+
+  if (head_ok) {
+    const int64_t slot = ((int64_t)b * p.Hq + head) * p.nsplit_max + split;
+    float* wo = p.ws_o + slot * D;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *(f32x4*)(wo + 16 * mt + 4 * g) = o[mt];
+    if (g == 0) {
+      p.ws_ml[slot * 2 + 0] = m_run;
+      p.ws_ml[slot * 2 + 1] = l_run;
+    }
+  }
+}
+
+// Combine the split partials: O = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s
+// (paged_attention.py:238-285 with the exponent in base 2).
+template <int DT, int D>
+__global__ __launch_bounds__(D) void paged_decode_combine_kernel(const DecodeParams p) {
+  const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int ctx = p.kv_len[b];
+  float acc = 0.0f;
+  if (ctx > 0) {
+    const int ns = (ctx + p.keys_per_split - 1) / p.keys_per_split;
+    const int64_t slot0 = ((int64_t)b * p.Hq + head) * p.nsplit_max;
+    float m = -__builtin_inff();
+    for (int s = 0; s < ns; ++s) m = fmaxf(m, p.ws_ml[(slot0 + s) * 2]);
+    float den = 0.0f;
+    for (int s = 0; s < ns; ++s) {
+      const float w = __builtin_amdgcn_exp2f(p.ws_ml[(slot0 + s) * 2] - m);
+      den += w * p.ws_ml[(slot0 + s) * 2 + 1];
+      acc += w * p.ws_o[(slot0 + s) * D + d];
+    }
+    acc /= den;
+  }
+  Elem<DT>::store1(p.o, (int64_t)b * p.o_sb + (int64_t)head * p.o_sh + d, acc);
+}
+
+int pick_keys_per_split(int B, int Hkv, int hchunks, int max_ctx) {
+  // enough work items to cover the chip several times over, but no smaller than 2 tiles
+  const int64_t units = (int64_t)B * Hkv * hchunks;
+  int kps = 512;
+  while (kps > 128 && units * ((max_ctx + kps - 1) / kps) < 4096) kps >>= 1;
+  return kps;
+}
+
+}  // namespace
+}  // namespace dlb
+
+extern "C" size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int page,
+                                            int max_blocks) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || page <= 0 || max_blocks <= 0) return 0;
+  const int group = Hq / Hkv;
+  const int hchunks = (group + 15) / 16;
+  const int64_t max_ctx = (int64_t)page * max_blocks;
+  if (max_ctx > 0x7fffffff) return 0;
+  const int kps = dlb::pick_keys_per_split(B, Hkv, hchunks, (int)max_ctx);
+  const int64_t ns = (max_ctx + kps - 1) / kps;
+  return (size_t)B * Hq * ns * (D + 2) * sizeof(float);
+}
+
+extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache,
+                                     void* o, const int32_t* block_table, const int32_t* kv_len,
+                                     int B, int Hq, int Hkv, int D, int page, int max_blocks,
+                                     int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page,
+                                     int64_t k_stride_tok, int64_t k_stride_head,
+                                     int64_t v_stride_page, int64_t v_stride_tok,
+                                     int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
+                                     int64_t bt_stride, float sm_scale, int dtype, void* ws,
+                                     size_t ws_bytes, void* stream) {
+  using namespace dlb;
+  if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || page < 1 || max_blocks < 1) return DLB_ERR_BAD_ARG;
+  if (Hq % Hkv != 0) return DLB_ERR_BAD_ARG;
+  if (B == 0) return DLB_OK;
+  if (!q || !k_cache || !v_cache || !o || !block_table || !kv_len) return DLB_ERR_BAD_ARG;
+  if (D != 64 && D != 128) return DLB_ERR_UNSUPPORTED;
+  if (page % 16 != 0) return DLB_ERR_UNSUPPORTED;
+  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
+  if ((int64_t)page * max_blocks > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
+  // 128-bit operand loads
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return DLB_ERR_UNSUPPORTED;
+  const int64_t strides[] = {q_stride_b,   q_stride_h,    k_stride_page, k_stride_tok,
+                             k_stride_head, v_stride_page, v_stride_tok,  v_stride_head};
+  for (int64_t sd : strides)
+    if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
+  const size_t need = dlb_paged_decode_ws_bytes(B, Hq, Hkv, D, page, max_blocks);
+  if (!ws || ws_bytes < need) return DLB_ERR_WORKSPACE;
+
+  DecodeParams p;
+  p.q = q;
+  p.k = k_cache;
+  p.v = v_cache;
+  p.o = o;
+  p.block_table = block_table;
+  p.kv_len = kv_len;
+  p.q_sb = q_stride_b;
+  p.q_sh = q_stride_h;
+  p.k_sp = k_stride_page;
+  p.k_st = k_stride_tok;
+  p.k_sh = k_stride_head;
+  p.v_sp = v_stride_page;
+  p.v_st = v_stride_tok;
+  p.v_sh = v_stride_head;
+  p.o_sb = o_stride_b;
+  p.o_sh = o_stride_h;
+  p.bt_stride = bt_stride;
+  p.B = B;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.group = Hq / Hkv;
+  p.hchunks = (p.group + 15) / 16;
+  p.page = page;
+  p.page_shift = -1;
+  for (int sh = 0; sh < 31; ++sh)
+    if ((1 << sh) == page) p.page_shift = sh;
+  p.max_blocks = max_blocks;
+  const int max_ctx = page * max_blocks;
+  p.keys_per_split = pick_keys_per_split(B, Hkv, p.hchunks, max_ctx);
+  p.nsplit_max = (max_ctx + p.keys_per_split - 1) / p.keys_per_split;
+  p.scale_log2e = sm_scale * 1.4426950408889634f;
+  p.ws_o = (float*)ws;
+  p.ws_ml = p.ws_o + (size_t)B * Hq * p.nsplit_max * D;
+
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid1((uint32_t)p.nsplit_max, (uint32_t)(Hkv * p.hchunks), (uint32_t)B);
+  const dim3 grid2((uint32_t)Hq, (uint32_t)B);
+#define DLB_LAUNCH_DECODE(DT_, D_)                                                              \
+  do {                                                                                          \
+    hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_>), grid1, dim3(64), 0, s, p);         \
+    hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p);       \
+  } while (0)
+  if (dtype == DLB_DTYPE_BF16) {
+    if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 128);
+    else DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 64);
+  } else {
+    if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
+    else DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 64);
+  }
+#undef DLB_LAUNCH_DECODE
+  return launch_status();
+}

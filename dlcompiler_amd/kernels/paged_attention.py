@@ -1,0 +1,81 @@
+"""``paged_attention_fwd`` with the signature of ``dlblas.kernels.paged_attention``
+(reference: python/dlBLAS/dlblas/kernels/paged_attention.py:492-671)."""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from .. import _lib
+
+
+def _as_int32(t: Tensor) -> Tensor:
+    return t if t.dtype == torch.int32 else t.to(torch.int32)
+
+
+def paged_attention_fwd(
+    q: Tensor,
+    k: Tensor,
+    v: Tensor,
+    o: Tensor,
+    block_offsets: Tensor,
+    q_start_loc: Tensor,
+    q_seqlens: Tensor,
+    kv_seqlens: Tensor,
+    max_seqlen: int,
+    window_size: int = None,
+    sm_scale: float = None,
+    logit_softcapping: float = None,
+):
+    """Paged attention forward, written into ``o``; returns ``None`` like the reference.
+
+    Args follow the reference: ``q`` [tokens, Hq, D]; ``k``/``v`` caches
+    [pages, page_size, Hkv, D]; ``block_offsets`` [batch, max_blocks] maps a sequence's
+    logical pages to physical ones; ``kv_seqlens`` [batch] context lengths.  The decode case
+    (one query token per sequence, ``q.shape[-3] == q_seqlens.size(0)``,
+    paged_attention.py:559) is implemented; sliding window and logit soft-capping are not.
+    """
+    _lib.require_cuda(q, k, v, o, block_offsets, kv_seqlens)
+    if window_size is not None and window_size > 0:
+        raise NotImplementedError("sliding-window paged attention is not implemented")
+    if logit_softcapping is not None and logit_softcapping > 0:
+        raise NotImplementedError("logit soft-capping is not implemented")
+    Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Lq == Lk, Lv == o.shape[-1]
+    if sm_scale is None:
+        sm_scale = 1.0 / (Lq**0.5)
+    batch, head = q_seqlens.shape[0], q.shape[-2]
+    is_decoding = q.shape[-3] == q_seqlens.size(0)
+    if not is_decoding:
+        raise NotImplementedError(
+            "only the decode branch (one query token per sequence) is implemented")
+    if Lv != Lk:
+        raise NotImplementedError("value head size must equal key head size")
+    assert k.dim() == 4 and v.dim() == 4 and k.shape[:3] == v.shape[:3]
+    assert q.dtype == k.dtype == v.dtype == o.dtype
+    num_kv_heads = k.shape[-2]
+    assert head % num_kv_heads == 0
+    page = k.size(1)
+    assert page >= 16
+    for t in (q, k, v, o):
+        assert t.stride(-1) == 1, "last dimension must be contiguous"
+    q3 = q.reshape(batch, head, Lq) if q.dim() != 3 else q
+    o3 = o.reshape(batch, head, Lv) if o.dim() != 3 else o
+    assert o3.data_ptr() == o.data_ptr()
+    block_offsets = _as_int32(block_offsets)
+    if block_offsets.stride(-1) != 1:
+        block_offsets = block_offsets.contiguous()
+    kv_seqlens = _as_int32(kv_seqlens).contiguous()
+    max_blocks = block_offsets.size(1)
+
+    lib = _lib.load()
+    ws_bytes = lib.dlb_paged_decode_ws_bytes(batch, head, num_kv_heads, Lq, page, max_blocks)
+    ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        st = lib.dlb_paged_decode_attn(
+            q3.data_ptr(), k.data_ptr(), v.data_ptr(), o3.data_ptr(), block_offsets.data_ptr(),
+            kv_seqlens.data_ptr(), batch, head, num_kv_heads, Lq, page, max_blocks,
+            q3.stride(0), q3.stride(1), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), o3.stride(0), o3.stride(1),
+            block_offsets.stride(0), float(sm_scale), _lib.torch_dtype_code(q.dtype),
+            ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(q.device))
+    _lib.check(st, "dlb_paged_decode_attn")

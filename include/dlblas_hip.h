@@ -90,6 +90,31 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
                              int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
                              void* ws, size_t ws_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Paged decode attention: one query token per sequence against a paged KV cache, GQA.
+ * Replaces the decode branch of paged_attention_fwd, kernels/paged_attention.py:604-671
+ * (_fwd_grouped_split_kernel :45-234 and _reduce_split_kernel :238-285).
+ *   q            [B, Hq, D]            strides q_stride_b, q_stride_h, unit last stride
+ *   k/v cache    [pages, page, Hkv, D] strides *_stride_page, *_stride_tok, *_stride_head
+ *   o            [B, Hq, D]            strides o_stride_b, o_stride_h
+ *   block_table  int32 [B, max_blocks] row stride bt_stride: physical page of logical page j
+ *   kv_len       int32 [B]             context length; rows with kv_len <= 0 produce zeros
+ * out[b, h] = softmax(q[b, h] . K[b, h / (Hq/Hkv)]^T * sm_scale) V, softmax in fp32 and P
+ * rounded to `dtype` before P.V, as in the reference.
+ * Supported: dtype bf16/f16, D in {64, 128}, page % 16 == 0, all strides multiples of 8 and
+ * base pointers 16-byte aligned.  ws: dlb_paged_decode_ws_bytes(...) bytes of device scratch
+ * (split-KV partials), caller-owned.
+ * ---------------------------------------------------------------------------------------- */
+size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int page, int max_blocks);
+int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, void* o,
+                          const int32_t* block_table, const int32_t* kv_len, int B, int Hq,
+                          int Hkv, int D, int page, int max_blocks, int64_t q_stride_b,
+                          int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_tok,
+                          int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_tok,
+                          int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
+                          int64_t bt_stride, float sm_scale, int dtype, void* ws,
+                          size_t ws_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

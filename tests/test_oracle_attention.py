@@ -1,0 +1,84 @@
+"""Pins oracle.attention (CPU) against torch's SDPA and closed-form cases."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import attention as oa
+
+
+def _rand(shape, seed, dtype=torch.bfloat16):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)).to(dtype)
+
+
+@pytest.mark.parametrize("hq,hkv", [(6, 6), (8, 2), (4, 1)])
+def test_prefill_matches_sdpa(hq, hkv):
+    lens = [5, 64, 1, 33]
+    total = sum(lens)
+    q, k, v = _rand((total, hq, 32), 0), _rand((total, hkv, 32), 1), _rand((total, hkv, 32), 2)
+    start = torch.tensor([0, 5, 69, 70], dtype=torch.int32)
+    o = oa.prefill_attention(q, k, v, start, torch.tensor(lens, dtype=torch.int32))
+    for s, l in zip(start.tolist(), lens):
+        ref = F.scaled_dot_product_attention(
+            q[s:s + l].float().transpose(0, 1)[None], k[s:s + l].float().transpose(0, 1)[None],
+            v[s:s + l].float().transpose(0, 1)[None], is_causal=True, enable_gqa=True)[0]
+        # only difference: the oracle rounds P to bf16 before P.V (as the reference does)
+        torch.testing.assert_close(o[s:s + l].float(), ref.transpose(0, 1), rtol=2e-2, atol=2e-2)
+
+
+def test_prefill_fp32_is_exactly_sdpa_semantics():
+    q, k, v = (_rand((40, 4, 16), i, torch.float32) for i in range(3))
+    o = oa.prefill_attention(q, k, v, torch.tensor([0, 17]), torch.tensor([17, 23]))
+    for s, l in [(0, 17), (17, 23)]:
+        ref = F.scaled_dot_product_attention(q[s:s + l].transpose(0, 1)[None],
+                                             k[s:s + l].transpose(0, 1)[None],
+                                             v[s:s + l].transpose(0, 1)[None], is_causal=True)[0]
+        torch.testing.assert_close(o[s:s + l], ref.transpose(0, 1), rtol=1e-5, atol=1e-6)
+
+
+def test_prefill_closed_forms():
+    # first token of every sequence attends only to itself -> output = its V row
+    q, k, v = _rand((12, 4, 16), 0), _rand((12, 2, 16), 1), _rand((12, 2, 16), 2)
+    o = oa.prefill_attention(q, k, v, torch.tensor([0, 7]), torch.tensor([7, 5]))
+    for s in (0, 7):
+        assert torch.equal(o[s], v[s].repeat_interleave(2, dim=0))
+    # identical keys -> uniform probabilities -> causal prefix mean of V
+    k2 = k[:1].expand(12, 2, 16).contiguous()
+    o2 = oa.prefill_attention(q, k2, v, torch.tensor([0]), torch.tensor([12]))
+    prefix = v.float().cumsum(0) / torch.arange(1, 13)[:, None, None]
+    torch.testing.assert_close(o2.float(), prefix.repeat_interleave(2, dim=1), rtol=2e-2, atol=2e-2)
+    # GQA mapping: query head h uses kv head h // group
+    v3 = torch.zeros_like(v)
+    v3[:, 1] = 1.0
+    o3 = oa.prefill_attention(q, k, v3, torch.tensor([0]), torch.tensor([12]))
+    assert (o3[:, :2] == 0).all() and (o3[:, 2:] == 1).all()
+
+
+def test_paged_decode_matches_dense_and_is_permutation_invariant():
+    lens = [1, 64, 65, 130, 17]
+    ks = [_rand((l, 2, 32), 10 + i) for i, l in enumerate(lens)]
+    vs = [_rand((l, 2, 32), 20 + i) for i, l in enumerate(lens)]
+    q = _rand((5, 8, 32), 3)
+    outs = []
+    for seed in (0, 1):
+        kc, vc, table = oa.make_paged_cache(ks, vs, page=16, num_pages=40, seed=seed)
+        outs.append(oa.paged_decode(q, kc, vc, table, torch.tensor(lens)))
+    assert torch.equal(outs[0], outs[1])                  # page placement does not matter
+    for b, l in enumerate(lens):
+        ref = F.scaled_dot_product_attention(q[b].float()[None, :, None, :],
+                                             ks[b].float().transpose(0, 1)[None],
+                                             vs[b].float().transpose(0, 1)[None],
+                                             enable_gqa=True)[0, :, 0]
+        torch.testing.assert_close(outs[0][b].float(), ref, rtol=2e-2, atol=2e-2)
+    assert torch.equal(outs[0][0], vs[0][0].repeat_interleave(4, dim=0))   # ctx = 1
+
+
+def test_paged_decode_zero_length_and_scale():
+    ks, vs = [_rand((20, 1, 16), 1)], [_rand((20, 1, 16), 2)]
+    kc, vc, table = oa.make_paged_cache(ks, vs, page=16)
+    q = _rand((1, 2, 16), 3)
+    assert (oa.paged_decode(q, kc, vc, table, torch.tensor([0])) == 0).all()
+    a = oa.paged_decode(q, kc, vc, table, torch.tensor([20]), sm_scale=0.0)
+    torch.testing.assert_close(a[0, 0].float(), vs[0][:, 0].float().mean(0), rtol=2e-2, atol=2e-2)
+    assert math.isfinite(a.float().sum().item())
