@@ -115,6 +115,27 @@ int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cach
                           int64_t bt_stride, float sm_scale, int dtype, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Varlen causal flash-attention prefill on packed sequences, GQA.
+ * Replaces context_attention_fwd + _fwd_kernel, kernels/prefill_attention.py:39-181.
+ *   q [tokens, Hq, D], k/v [tokens, Hkv, D], o [tokens, Hq, D]; token and head strides given,
+ *   unit stride in D.  Sequence s owns tokens start_loc[s] .. start_loc[s] + seq_len[s] - 1
+ *   (int32 [B] each; with cu_seqlens: start_loc = cu[:-1], seq_len = cu[1:] - cu[:-1]).
+ *   max_len >= max(seq_len) sizes the grid (the reference's max_input_len).
+ * o[t, h] = sum_{t' <= t, same sequence} softmax_t'(q[t, h] . k[t', h / (Hq/Hkv)] * sm_scale)
+ *           v[t', h / (Hq/Hkv)], softmax in fp32, P rounded to `dtype` before P.V.
+ * (The reference fixes sm_scale = 1/sqrt(D); pass that for drop-in behaviour.)
+ * Supported: dtype bf16/f16, D in {64, 128}, q/k/v strides multiples of 8 and bases 16-byte
+ * aligned, o strides multiples of 4 and base 8-byte aligned.  Tokens outside every sequence
+ * are not written.
+ * ---------------------------------------------------------------------------------------- */
+int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o,
+                            const int32_t* start_loc, const int32_t* seq_len, int B, int Hq,
+                            int Hkv, int D, int max_len, int64_t q_stride_tok,
+                            int64_t q_stride_head, int64_t k_stride_tok, int64_t k_stride_head,
+                            int64_t v_stride_tok, int64_t v_stride_head, int64_t o_stride_tok,
+                            int64_t o_stride_head, float sm_scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
