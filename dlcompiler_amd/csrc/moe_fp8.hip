@@ -1,0 +1,487 @@
+// fp8 (OCP e4m3fn) fused-MoE building blocks for gfx950:
+//   * per-token-group activation quantisation (groups of 128 along K, fp32 scales);
+//   * expert-grouped GEMM over block-aligned routing (64-row blocks, one expert per block) on
+//     the 16x16x128 f8f6f4 MFMA, with the block scales applied per 128-deep K chunk:
+//         acc += mfma(x_q[:, kc], w_q[:, kc]) * x_scale[row, kc] * w_scale[n / 128, kc]
+//     in two flavours -- "gate_up" (A rows gathered by token, SiLU-and-mul and re-quantisation
+//     of the intermediate fused into the epilogue) and "down" (routing weight applied, rows
+//     scattered back to their (token, slot) position);
+//   * the deterministic sum over the top-k slots.
+//
+// Pipeline shape and layouts follow the reference's bf16 fused_moe
+// (python/dlBLAS/dlblas/kernels/fused_moe.py:296-376: sort by expert, grouped GEMM over
+// w1 [E, 2I, H] with the gate rows first, activation, grouped GEMM over w2 [E, H, I] times
+// the routing weight, sum over top-k; kernel :82-175).  The fp8 scheme itself has no
+// counterpart there; its nearest precedent is the int8 per-token quantisation and
+// scale-in-epilogue GEMM of python/dlBLAS/dlblas/kernels/w8a8.py:102-106,275-335.
+//
+// GEMM mapping.  The MFMA runs "transposed": weight rows are the A operand (M index = output
+// column n), activations the B operand (N index = token row), so a lane's four accumulator
+// registers are four consecutive n of ONE token: the activation scale is a per-lane scalar
+// and the epilogues store 4 adjacent outputs.  Weight fragments go straight from HBM/L2 into
+// operand registers (each wave owns its own n range, so nothing is shared between waves);
+// only the 64 x 128-byte activation chunk is staged through LDS, double-buffered.
+#include "common.h"
+
+namespace dlb {
+namespace {
+
+constexpr float kFp8Max = 448.0f;
+constexpr float kQuantEps = 1e-10f;
+
+__device__ __forceinline__ unsigned int pack4_fp8(float a, float b, float c, float d) {
+  // v_cvt_pk_fp8_f32 rounds to nearest even; values beyond +-464 would become NaN, so clamp.
+  a = fminf(fmaxf(a, -kFp8Max), kFp8Max);
+  b = fminf(fmaxf(b, -kFp8Max), kFp8Max);
+  c = fminf(fmaxf(c, -kFp8Max), kFp8Max);
+  d = fminf(fmaxf(d, -kFp8Max), kFp8Max);
+  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  return (unsigned int)r;
+}
+
+// ---------------------------------------------------------------------------------------
+// per-token-group quantisation: one DPP row (16 lanes x 8 elements) per 128-element group
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void quant_fp8_group128_kernel(
+    const unsigned short* __restrict__ x, unsigned char* __restrict__ xq, float* __restrict__ xs,
+    int64_t total_groups, int groups_per_row, int64_t ldx, int64_t ldq, int64_t lds) {
+  const int lane16 = threadIdx.x & 15;
+  const int64_t gidx = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = gidx < total_groups;
+  const int64_t row = live ? gidx / groups_per_row : 0;
+  const int gc = live ? (int)(gidx - row * groups_per_row) : 0;
+  u32x4 raw = u32x4{0u, 0u, 0u, 0u};
+  if (live) raw = *(const u32x4*)(x + row * ldx + gc * 128 + lane16 * 8);
+  float v[8];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    v[2 * w] = Elem<DT>::lo(raw[w]);
+    v[2 * w + 1] = Elem<DT>::hi(raw[w]);
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+  amax = row16_max(amax);
+  const float scale = fmaxf(amax, kQuantEps) / kFp8Max;
+  if (live) {
+    u32x2 q;
+    q[0] = pack4_fp8(v[0] / scale, v[1] / scale, v[2] / scale, v[3] / scale);
+    q[1] = pack4_fp8(v[4] / scale, v[5] / scale, v[6] / scale, v[7] / scale);
+    *(u32x2*)(xq + row * ldq + gc * 128 + lane16 * 8) = q;
+    if (lane16 == 0) xs[row * lds + gc] = scale;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// grouped GEMM
+// ---------------------------------------------------------------------------------------
+struct MoeGemmParams {
+  const unsigned char* a;     // activations fp8 [rows, K]
+  const float* a_scale;       // [rows, K / 128]
+  const unsigned char* w;     // weights fp8 [E_local, N, K]
+  const float* w_scale;       // [E_local, N / 128, K / 128]
+  const int32_t* sorted_ids;  // [num_mblocks * 64]
+  const int32_t* expert_ids;  // [num_mblocks]
+  int num_mblocks, num_ntiles, grid_real;
+  int K, N, KC;               // KC = K / 128
+  int topk, numel;            // flat slots = tokens * topk (also the pad sentinel)
+  int num_tokens;
+  int expert_offset;          // weights hold experts [expert_offset, expert_offset + E_local)
+  int num_local;              // E_local
+  // gate_up flavour
+  unsigned char* hq;          // [num_mblocks * 64, I]
+  float* hs;                  // [num_mblocks * 64, I / 128]
+  int I;
+  // down flavour
+  void* out;                  // [numel, N] bf16/f16
+  const float* topk_w;        // [numel]
+};
+
+constexpr int kBM = 64;         // rows (routing slots) per workgroup = alignment block
+constexpr int kARow = 128 + 16; // LDS row pitch of the activation chunk (bytes)
+
+__device__ __forceinline__ f32x4 mfma_fp8(const i32x8& a, const i32x8& b) {
+  const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled opcode
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, z, 0, 0, 0, 0, 0, 0);
+}
+
+// GATED = true : gate_up GEMM (N = 2I), tile = 128 gate cols + the matching 128 up cols,
+//                epilogue silu(gate) * up -> fp8 + per-128 scale, rows kept in sorted order.
+// GATED = false: down GEMM, tile = 256 cols, epilogue * routing weight -> out[slot, n].
+template <bool GATED, int DT>
+__global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][kBM * kARow];
+  __shared__ __attribute__((aligned(16))) float as_lds[2][kBM];
+  __shared__ float red_lds[4][kBM];
+  __shared__ int32_t sid_lds[kBM];
+
+  // workgroups are dealt round-robin to the 8 XCDs; undo that so that neighbours in the
+  // logical order (same n tile, consecutive row blocks = mostly the same expert) share an L2
+  const int per_xcd = gridDim.x >> 3;
+  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= p.grid_real) return;
+  const int mb = logical % p.num_mblocks;
+  const int nt = logical / p.num_mblocks;
+  const int e_global = p.expert_ids[mb];
+  const int e = e_global - p.expert_offset;
+  if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int row0 = mb * kBM;
+  const int K = p.K, KC = p.KC;
+
+  if (tid < kBM) sid_lds[tid] = p.sorted_ids[row0 + tid];
+
+  // ---- activation chunk staging: thread -> (row = tid / 4, 32-byte segment = tid % 4)
+  const int arow = tid >> 2, aseg = tid & 3;
+  const unsigned char* a_ptr;
+  const float* as_ptr;
+  {
+    int64_t src_row;
+    if (GATED) {
+      const int sid = p.sorted_ids[row0 + arow];
+      src_row = min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
+    } else {
+      src_row = row0 + arow;
+    }
+    a_ptr = p.a + src_row * K + aseg * 32;
+    as_ptr = p.a_scale + src_row * KC;
+  }
+
+  // ---- weight fragments: sub-tile j of this wave covers 16 output columns
+  int ncol[4];   // first column of sub-tile j in the expert's [N, K] matrix
+  int sblk[4];   // its 128-row scale block
+  if (GATED) {
+    const int n0 = nt * 128 + wave * 32;
+    ncol[0] = n0;
+    ncol[1] = n0 + 16;
+    ncol[2] = p.I + n0;
+    ncol[3] = p.I + n0 + 16;
+  } else {
+    const int n0 = nt * 256 + wave * 64;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ncol[j] = n0 + 16 * j;
+  }
+  const unsigned char* w_ptr[4];
+  const float* ws_ptr[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    sblk[j] = min(ncol[j] >> 7, (p.N >> 7) - 1);
+    // lanes of group g take K bytes [16g, 16g+16) and [64+16g, 64+16g+16) of each chunk
+    const int n = min(ncol[j] + c, p.N - 1);
+    w_ptr[j] = p.w + ((int64_t)e * p.N + n) * K + 16 * g;
+    ws_ptr[j] = p.w_scale + ((int64_t)e * (p.N >> 7) + sblk[j]) * KC;
+  }
+
+  f32x4 acc[4][4];  // [token sub-tile mt][column sub-tile j]
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 areg[2];
+  float asreg = 0.0f;
+  i32x8 breg[2][4];
+  float bsreg[2][4];
+
+  auto load_a = [&](int kc) {
+    areg[0] = *(const u32x4*)(a_ptr + kc * 128);
+    areg[1] = *(const u32x4*)(a_ptr + kc * 128 + 16);
+    if (aseg == 0) asreg = as_ptr[kc];
+  };
+  auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const u32x4 lo = *(const u32x4*)(w_ptr[j] + kc * 128);
+      const u32x4 hi = *(const u32x4*)(w_ptr[j] + kc * 128 + 64);
+      b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+                   (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      bs[j] = ws_ptr[j][kc];
+    }
+  };
+  auto store_a = [&](int buf) {
+    unsigned char* dst = a_lds[buf] + arow * kARow + aseg * 32;
+    *(u32x4*)(dst) = areg[0];
+    *(u32x4*)(dst + 16) = areg[1];
+    if (aseg == 0) as_lds[buf][arow] = asreg;
+  };
+  auto compute = [&](int buf, const i32x8 (&b)[4], const float (&bs)[4]) {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const unsigned char* src = a_lds[buf] + (16 * mt + c) * kARow + 16 * g;
+      const u32x4 lo = *(const u32x4*)(src);
+      const u32x4 hi = *(const u32x4*)(src + 64);
+      const i32x8 x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+                            (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      const float as = as_lds[buf][16 * mt + c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 part = mfma_fp8(b[j], x);
+        const float sc = as * bs[j];
+        acc[mt][j] += part * sc;
+      }
+    }
+  };
+
+  load_a(0);
+  load_b(0, breg[0], bsreg[0]);
+  for (int kc = 0; kc < KC; kc += 2) {
+    // even chunk: buffers 0
+    store_a(0);
+    __syncthreads();
+    if (kc + 1 < KC) {
+      load_a(kc + 1);
+      load_b(kc + 1, breg[1], bsreg[1]);
+    }
+    compute(0, breg[0], bsreg[0]);
+    if (kc + 1 < KC) {
+      // odd chunk: buffers 1
+      store_a(1);
+      __syncthreads();
+      if (kc + 2 < KC) {
+        load_a(kc + 2);
+        load_b(kc + 2, breg[0], bsreg[0]);
+      }
+      compute(1, breg[1], bsreg[1]);
+    }
+  }
+
+  // ---- epilogues: lane holds token (16*mt + c), columns ncol[j] + 4*g + i
+  if (GATED) {
+    float h[4][2][4];
+    float amax[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      amax[mt] = 0.0f;
+#pragma unroll
+      for (int jg = 0; jg < 2; ++jg) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float gate = acc[mt][jg][i];
+          const float up = acc[mt][jg + 2][i];
+          const float v = gate / (1.0f + __expf(-gate)) * up;
+          h[mt][jg][i] = v;
+          amax[mt] = fmaxf(amax[mt], fabsf(v));
+        }
+      }
+      amax[mt] = fmaxf(amax[mt], __shfl_xor(amax[mt], 16));
+      amax[mt] = fmaxf(amax[mt], __shfl_xor(amax[mt], 32));
+      if (g == 0) red_lds[wave][16 * mt + c] = amax[mt];
+    }
+    __syncthreads();
+    const int scol = nt;  // 128-column group index of the intermediate
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int r = 16 * mt + c;
+      const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
+      const float scale = fmaxf(m, kQuantEps) / kFp8Max;
+      const int64_t orow = row0 + r;
+#pragma unroll
+      for (int jg = 0; jg < 2; ++jg) {
+        const unsigned int q = pack4_fp8(h[mt][jg][0] / scale, h[mt][jg][1] / scale,
+                                         h[mt][jg][2] / scale, h[mt][jg][3] / scale);
+        *(unsigned int*)(p.hq + orow * p.I + nt * 128 + wave * 32 + 16 * jg + 4 * g) = q;
+      }
+      if (wave == 0 && g == 0) p.hs[orow * (p.I >> 7) + scol] = scale;
+    }
+  } else {
+    __syncthreads();  // sid_lds visible (also true after the main loop's barriers)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int sid = sid_lds[16 * mt + c];
+      if (sid < p.numel) {
+        const float rw = p.topk_w[sid];
+        unsigned short* orow = (unsigned short*)p.out + (int64_t)sid * p.N;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = ncol[j] + 4 * g;
+          if (n < p.N) {
+            u32x2 o2;
+            o2[0] = Elem<DT>::pack(acc[mt][j][0] * rw, acc[mt][j][1] * rw);
+            o2[1] = Elem<DT>::pack(acc[mt][j][2] * rw, acc[mt][j][3] * rw);
+            *(u32x2*)(orow + n) = o2;
+          }
+        }
+      }
+    }
+  }
+}
+
+// out[t, n] = sum_j in[t * topk + j, n], fp32 accumulation in slot order, one rounding
+template <int DT>
+__global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restrict__ in,
+                                                           u32x4* __restrict__ out,
+                                                           int64_t total_vec, int vec_per_row,
+                                                           int topk) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total_vec) return;
+  const int64_t t = i / vec_per_row;
+  const int col = (int)(i - t * vec_per_row);
+  float s[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) s[q] = 0.0f;
+  for (int j = 0; j < topk; ++j) {
+    const u32x4 v = __builtin_nontemporal_load(in + (t * topk + j) * vec_per_row + col);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      s[2 * w] += Elem<DT>::lo(v[w]);
+      s[2 * w + 1] += Elem<DT>::hi(v[w]);
+    }
+  }
+  u32x4 r;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) r[w] = Elem<DT>::pack(s[2 * w], s[2 * w + 1]);
+  out[i] = r;
+}
+
+int check_gemm_common(const void* a, const void* a_scale, const void* w, const void* w_scale,
+                      const void* sorted_ids, const void* expert_ids, int num_mblocks, int K,
+                      int N) {
+  if (num_mblocks < 0 || K < 1 || N < 1) return DLB_ERR_BAD_ARG;
+  if (num_mblocks == 0) return DLB_OK;
+  if (!a || !a_scale || !w || !w_scale || !sorted_ids || !expert_ids) return DLB_ERR_BAD_ARG;
+  if (K % 128 != 0 || N % 128 != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(a) || !aligned16(w)) return DLB_ERR_UNSUPPORTED;
+  return DLB_OK;
+}
+
+}  // namespace
+}  // namespace dlb
+
+extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
+                                             int K, int64_t ld_x, int64_t ld_q, int64_t ld_s,
+                                             int dtype, void* stream) {
+  using namespace dlb;
+  if (M < 0 || K < 0 || ld_x < K || ld_q < K || ld_s < K / 128) return DLB_ERR_BAD_ARG;
+  if (M == 0 || K == 0) return DLB_OK;
+  if (!x || !xq || !xs) return DLB_ERR_BAD_ARG;
+  if (K % 128 != 0 || ld_x % 8 != 0 || ld_q % 8 != 0 || !aligned16(x) ||
+      (reinterpret_cast<uintptr_t>(xq) & 7u) != 0)
+    return DLB_ERR_UNSUPPORTED;
+  const int gpr = K / 128;
+  const int64_t total = M * gpr;
+  const dim3 grid((uint32_t)ceil_div(total, 16));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DLB_DTYPE_BF16)
+    hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_BF16>, grid, dim3(256), 0, s,
+                       (const unsigned short*)x, (unsigned char*)xq, xs, total, gpr, ld_x, ld_q,
+                       ld_s);
+  else if (dtype == DLB_DTYPE_F16)
+    hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_F16>, grid, dim3(256), 0, s,
+                       (const unsigned short*)x, (unsigned char*)xq, xs, total, gpr, ld_x, ld_q,
+                       ld_s);
+  else
+    return DLB_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
+extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q,
+                                        const float* w1s, const int32_t* sorted_ids,
+                                        const int32_t* expert_ids, int num_mblocks,
+                                        int num_tokens, int topk, int H, int I,
+                                        int expert_offset, int num_local_experts, void* hq,
+                                        float* hs, void* stream) {
+  using namespace dlb;
+  const int st = check_gemm_common(xq, xs, w1q, w1s, sorted_ids, expert_ids, num_mblocks, H, I);
+  if (st != DLB_OK || num_mblocks == 0) return st;
+  if (num_tokens < 1 || topk < 1 || num_local_experts < 1 || !hq || !hs) return DLB_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(hq) & 3u) != 0) return DLB_ERR_UNSUPPORTED;
+  MoeGemmParams p = {};
+  p.a = (const unsigned char*)xq;
+  p.a_scale = xs;
+  p.w = (const unsigned char*)w1q;
+  p.w_scale = w1s;
+  p.sorted_ids = sorted_ids;
+  p.expert_ids = expert_ids;
+  p.num_mblocks = num_mblocks;
+  p.num_ntiles = I / 128;
+  p.K = H;
+  p.N = 2 * I;
+  p.KC = H / 128;
+  p.topk = topk;
+  p.numel = num_tokens * topk;
+  p.num_tokens = num_tokens;
+  p.expert_offset = expert_offset;
+  p.num_local = num_local_experts;
+  p.hq = (unsigned char*)hq;
+  p.hs = hs;
+  p.I = I;
+  p.grid_real = p.num_mblocks * p.num_ntiles;
+  const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
+  hipLaunchKernelGGL((moe_gemm_fp8_kernel<true, DLB_DTYPE_BF16>), dim3(grid), dim3(256), 0,
+                     (hipStream_t)stream, p);
+  return launch_status();
+}
+
+extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q,
+                                     const float* w2s, const int32_t* sorted_ids,
+                                     const int32_t* expert_ids, const float* topk_weights,
+                                     int num_mblocks, int num_tokens, int topk, int H, int I,
+                                     int expert_offset, int num_local_experts, void* out,
+                                     int out_dtype, void* stream) {
+  using namespace dlb;
+  const int st = check_gemm_common(hq, hs, w2q, w2s, sorted_ids, expert_ids, num_mblocks, I, H);
+  if (st != DLB_OK || num_mblocks == 0) return st;
+  if (num_tokens < 1 || topk < 1 || num_local_experts < 1 || !out || !topk_weights)
+    return DLB_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(out) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  MoeGemmParams p = {};
+  p.a = (const unsigned char*)hq;
+  p.a_scale = hs;
+  p.w = (const unsigned char*)w2q;
+  p.w_scale = w2s;
+  p.sorted_ids = sorted_ids;
+  p.expert_ids = expert_ids;
+  p.num_mblocks = num_mblocks;
+  p.num_ntiles = (int)ceil_div(H, 256);
+  p.K = I;
+  p.N = H;
+  p.KC = I / 128;
+  p.topk = topk;
+  p.numel = num_tokens * topk;
+  p.num_tokens = num_tokens;
+  p.expert_offset = expert_offset;
+  p.num_local = num_local_experts;
+  p.out = out;
+  p.topk_w = topk_weights;
+  p.I = I;
+  p.grid_real = p.num_mblocks * p.num_ntiles;
+  const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
+  if (out_dtype == DLB_DTYPE_BF16)
+    hipLaunchKernelGGL((moe_gemm_fp8_kernel<false, DLB_DTYPE_BF16>), dim3(grid), dim3(256), 0,
+                       (hipStream_t)stream, p);
+  else if (out_dtype == DLB_DTYPE_F16)
+    hipLaunchKernelGGL((moe_gemm_fp8_kernel<false, DLB_DTYPE_F16>), dim3(grid), dim3(256), 0,
+                       (hipStream_t)stream, p);
+  else
+    return DLB_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
+extern "C" int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk,
+                                int64_t N, int dtype, void* stream) {
+  using namespace dlb;
+  if (num_tokens < 0 || topk < 1 || N < 0) return DLB_ERR_BAD_ARG;
+  if (num_tokens == 0 || N == 0) return DLB_OK;
+  if (!in || !out) return DLB_ERR_BAD_ARG;
+  if (N % 8 != 0 || !aligned16(in) || !aligned16(out)) return DLB_ERR_UNSUPPORTED;
+  const int64_t total = num_tokens * (N / 8);
+  const dim3 grid((uint32_t)ceil_div(total, 256));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DLB_DTYPE_BF16)
+    hipLaunchKernelGGL(moe_topk_sum_kernel<DLB_DTYPE_BF16>, grid, dim3(256), 0, s,
+                       (const u32x4*)in, (u32x4*)out, total, (int)(N / 8), topk);
+  else if (dtype == DLB_DTYPE_F16)
+    hipLaunchKernelGGL(moe_topk_sum_kernel<DLB_DTYPE_F16>, grid, dim3(256), 0, s,
+                       (const u32x4*)in, (u32x4*)out, total, (int)(N / 8), topk);
+  else
+    return DLB_ERR_UNSUPPORTED;
+  return launch_status();
+}

@@ -1,0 +1,125 @@
+"""Fused MoE MLP operators, mirroring ``dlblas.kernels.fused_moe``
+(reference: python/dlBLAS/dlblas/kernels/fused_moe.py:238-376).
+
+``fused_moe_fp8`` / ``per_token_group_quant_fp8`` are this package's own names: the reference
+has no fp8 path; they keep the argument order and weight layouts of ``fused_moe``
+(``w1 [E, 2I, H]`` with the gate rows first, ``w2 [E, H, I]``).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from .moe_gating import moe_align_block_size
+
+_ALIGN_BLOCK = 64  # rows per grouped-GEMM workgroup
+
+
+def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
+    """x [M, K] bf16/f16 -> (xq float8_e4m3fn [M, K], xs fp32 [M, K // 128]).
+
+    Per group of 128 along K: ``scale = max(absmax, 1e-10) / 448``,
+    ``q = rne(clamp(x / scale, -448, 448))``.
+    """
+    if group_size != 128:
+        raise NotImplementedError("only groups of 128 are implemented")
+    assert x.dim() == 2
+    _lib.require_cuda(x)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    M, K = x.shape
+    if K % 128 != 0:
+        raise ValueError("K must be a multiple of 128")
+    xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=x.device)
+    xs = torch.empty((M, K // 128), dtype=torch.float32, device=x.device)
+    if M > 0:
+        lib = _lib.load()
+        with torch.cuda.device(x.device):
+            st = lib.dlb_per_token_group_quant_fp8(
+                x.data_ptr(), xq.data_ptr(), xs.data_ptr(), M, K, x.stride(0) if M > 1 else K, K,
+                K // 128, _lib.torch_dtype_code(x.dtype), _lib.current_stream_ptr(x.device))
+        _lib.check(st, "dlb_per_token_group_quant_fp8")
+    return xq, xs
+
+
+def get_start_end(topk_idx: torch.Tensor, sorted_idx: torch.Tensor, num_experts: int):
+    """``(exp_start, exp_end)`` of each expert's run in the expert-sorted slot list
+    (reference: fused_moe.py:267-293; ``end = cumsum(counts)``, ``start = end - counts``).
+    ``sorted_idx`` only fixes the dtype/device of the result, as in the reference."""
+    _, _, _, counts = moe_align_block_size(topk_idx, 1, num_experts, return_counts=True)
+    exp_end = counts.to(sorted_idx.dtype).cumsum(0).to(sorted_idx.dtype)
+    exp_start = exp_end - counts.to(sorted_idx.dtype)
+    return exp_start, exp_end
+
+
+def fused_moe_fp8(hidden_states: torch.Tensor,
+                  w1_q: torch.Tensor,
+                  w1_s: torch.Tensor,
+                  w2_q: torch.Tensor,
+                  w2_s: torch.Tensor,
+                  topk_weights: torch.Tensor,
+                  topk_ids: torch.Tensor,
+                  topk: int,
+                  expert_offset: int = 0,
+                  num_experts: int = None,
+                  renormalize: bool = False) -> torch.Tensor:
+    """fp8 MoE MLP: per-token-group quant -> gate_up grouped GEMM (+SiLU-and-mul, re-quant)
+    -> down grouped GEMM (x routing weight) -> sum over the top-k slots.
+
+    ``hidden_states`` [T, H] bf16/f16; ``w1_q`` [E, 2I, H] / ``w2_q`` [E, H, I]
+    float8_e4m3fn with fp32 scales per 128x128 block (``w1_s`` [E, 2I/128, H/128],
+    ``w2_s`` [E, H/128, I/128]); ``topk_weights``/``topk_ids`` [T, topk].  ``E`` is the
+    number of local experts, holding global experts ``expert_offset .. expert_offset + E``;
+    ``num_experts`` the global count (defaults to ``E``), as in the reference.
+    """
+    _lib.require_cuda(hidden_states, w1_q, w1_s, w2_q, w2_s, topk_weights, topk_ids)
+    assert hidden_states.dim() == 2 and topk_ids.shape == topk_weights.shape
+    T, H = hidden_states.shape
+    E, N2, H1 = w1_q.shape
+    I = N2 // 2
+    assert H1 == H and w2_q.shape == (E, H, I) and topk_ids.shape == (T, topk)
+    assert w1_q.dtype == torch.float8_e4m3fn and w2_q.dtype == torch.float8_e4m3fn
+    assert w1_q.is_contiguous() and w2_q.is_contiguous()
+    assert w1_s.shape == (E, N2 // 128, H // 128) and w2_s.shape == (E, H // 128, I // 128)
+    if num_experts is None:
+        num_experts = E
+    dev = hidden_states.device
+    dt = hidden_states.dtype
+    if T == 0:
+        return hidden_states.new_empty((0, H))
+
+    if renormalize:
+        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+    topk_weights = topk_weights.to(torch.float32).contiguous()
+    w1_s = w1_s.to(torch.float32).contiguous()
+    w2_s = w2_s.to(torch.float32).contiguous()
+
+    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, _ALIGN_BLOCK, num_experts)
+    num_mblocks = expert_ids.numel()
+    xq, xs = per_token_group_quant_fp8(hidden_states)
+
+    rows = num_mblocks * _ALIGN_BLOCK
+    hq = torch.empty((rows, I), dtype=torch.float8_e4m3fn, device=dev)
+    hs = torch.empty((rows, I // 128), dtype=torch.float32, device=dev)
+    full = (expert_offset == 0 and num_experts == E)
+    slots = (torch.empty if full else torch.zeros)((T * topk, H), dtype=dt, device=dev)
+    out = torch.empty((T, H), dtype=dt, device=dev)
+
+    lib = _lib.load()
+    stream = _lib.current_stream_ptr(dev)
+    with torch.cuda.device(dev):
+        st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
+                                          w1_s.data_ptr(), sorted_ids.data_ptr(),
+                                          expert_ids.data_ptr(), num_mblocks, T, topk, H, I,
+                                          expert_offset, E, hq.data_ptr(), hs.data_ptr(), stream)
+        _lib.check(st, "dlb_moe_gemm_fp8_gate_up")
+        st = lib.dlb_moe_gemm_fp8_down(hq.data_ptr(), hs.data_ptr(), w2_q.data_ptr(),
+                                       w2_s.data_ptr(), sorted_ids.data_ptr(),
+                                       expert_ids.data_ptr(), topk_weights.data_ptr(),
+                                       num_mblocks, T, topk, H, I, expert_offset, E,
+                                       slots.data_ptr(), _lib.torch_dtype_code(dt), stream)
+        _lib.check(st, "dlb_moe_gemm_fp8_down")
+        st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), T, topk, H,
+                                  _lib.torch_dtype_code(dt), stream)
+        _lib.check(st, "dlb_moe_topk_sum")
+    return out

@@ -136,6 +136,52 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
                             int64_t v_stride_tok, int64_t v_stride_head, int64_t o_stride_tok,
                             int64_t o_stride_head, float sm_scale, int dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * fp8 fused-MoE building blocks (OCP e4m3fn, fp32 scales per 128 along K; weights carry one
+ * scale per 128 x 128 block).  Pipeline shape follows fused_moe, kernels/fused_moe.py:296-376
+ * (grouped GEMM kernel :82-175); the fp8 scheme has no reference counterpart -- nearest
+ * precedent: per-token int8 quant and scale-in-epilogue GEMM, kernels/w8a8.py:102-106,275-335.
+ *
+ * Quantisation rule (activations and the intermediate): for each group of 128 consecutive
+ * elements of a row, scale = max(absmax, 1e-10) / 448 and q = rne_e4m3(clamp(x / scale, +-448)).
+ * ---------------------------------------------------------------------------------------- */
+
+/* x [M, K] bf16/f16 (row stride ld_x) -> xq [M, K] fp8 (row stride ld_q, bytes),
+ * xs [M, K/128] fp32 (row stride ld_s).  K % 128 == 0. */
+int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M, int K,
+                                  int64_t ld_x, int64_t ld_q, int64_t ld_s, int dtype,
+                                  void* stream);
+
+/* gate_up grouped GEMM + SiLU-and-mul + re-quantisation.
+ *   xq [num_tokens, H] fp8, xs [num_tokens, H/128]
+ *   w1q [num_local_experts, 2I, H] fp8 (gate rows first), w1s [num_local_experts, 2I/128, H/128]
+ *   sorted_ids [num_mblocks * 64], expert_ids [num_mblocks]: output of
+ *     dlb_moe_align_block_size with block = 64 (flat slot = token * topk + j, sentinel
+ *     num_tokens * topk, expert -1 for unused blocks); blocks whose expert lies outside
+ *     [expert_offset, expert_offset + num_local_experts) are skipped
+ *   hq [num_mblocks * 64, I] fp8 and hs [num_mblocks * 64, I/128]: row r holds
+ *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r
+ * H % 128 == 0, I % 128 == 0. */
+int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q, const float* w1s,
+                             const int32_t* sorted_ids, const int32_t* expert_ids,
+                             int num_mblocks, int num_tokens, int topk, int H, int I,
+                             int expert_offset, int num_local_experts, void* hq, float* hs,
+                             void* stream);
+
+/* down grouped GEMM: out[slot, :] = (h_r W_down^T) * topk_weights[slot] for every real slot
+ * (pad rows are skipped), out [num_tokens * topk, H] bf16/f16;
+ * w2q [num_local_experts, H, I] fp8, w2s [num_local_experts, H/128, I/128]. */
+int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q, const float* w2s,
+                          const int32_t* sorted_ids, const int32_t* expert_ids,
+                          const float* topk_weights, int num_mblocks, int num_tokens, int topk,
+                          int H, int I, int expert_offset, int num_local_experts, void* out,
+                          int out_dtype, void* stream);
+
+/* out[t, :] = sum_j in[t * topk + j, :] (fp32 accumulation in slot order, one rounding);
+ * replaces intermediate_cache2.sum(dim=1), kernels/fused_moe.py:375.  N % 8 == 0. */
+int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk, int64_t N,
+                     int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
