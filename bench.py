@@ -1,0 +1,431 @@
+#!/usr/bin/env python3
+"""Benchmark of the dlBLAS inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Runs the five BASELINE.json configurations (fused silu_and_mul, MoE gating + alignment,
+varlen causal prefill attention, paged decode attention, fp8 fused-MoE MLP) on synthetic,
+seeded inputs that are resident in HBM before the timed region, and prints ONE JSON line.
+A "step" is one call of an operator's public entry point on one batch.  The top-level
+`metric`/`value`/`roofline`/`cpu_baseline` describe the primary workload (--workload, default
+the fp8 fused MoE); `workloads` carries the same figures for every configuration.
+
+For each workload:
+  value      algorithmic work / wall time of K back-to-back steps (events on the launch stream)
+  roofline   the dominant kernel: algorithmic bytes (or FLOPs) per launch / its average launch
+             duration, measured with events bracketing that kernel inside the timed loop;
+             `traffic` (HBM bytes per launch from rocprofv3 --pmc) is read from
+             profiles/hbm_traffic.json when a measurement has been committed, else null
+  cpu_baseline  the CPU oracle (a port of the reference's PyTorch ground truth) timed on a
+             bounded sample of the same workload on this host's cores
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_FP8_TFLOPS = 5000.0
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+class Timer:
+    """Events on the current (launch) stream."""
+
+    def __init__(self):
+        self.pairs = []
+
+    def start(self):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        return ev
+
+    def stop(self, ev0):
+        ev1 = torch.cuda.Event(enable_timing=True)
+        ev1.record()
+        self.pairs.append((ev0, ev1))
+
+    def mean_ms(self):
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in self.pairs) / max(len(self.pairs), 1)
+
+
+def _time_steps(step, steps, warmup):
+    """step(i) launches one step; returns (ms_per_step over the whole region, per-step mean)."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t_all = Timer()
+    t_each = Timer()
+    ev = t_all.start()
+    for i in range(steps):
+        e = t_each.start()
+        step(i)
+        t_each.stop(e)
+    t_all.stop(ev)
+    torch.cuda.synchronize()
+    return t_all.mean_ms() / steps, t_each.mean_ms()
+
+
+def _traffic(name):
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(name)
+    except (OSError, ValueError):
+        return None
+
+
+# --------------------------------------------------------------------------------------
+# workloads
+# --------------------------------------------------------------------------------------
+def wl_silu(dev, steps, warmup, cpu):
+    from dlcompiler_amd.kernels.activation import silu_and_mul
+
+    M, N = 8192, 11008
+    nbuf = 3  # rotate > 2 x 256 MB of distinct buffers so nothing is served from cache
+    x0 = torch.randn((M, 2 * N), generator=_gen(0)).bfloat16()
+    xs = [x0.to(dev)] + [x0.to(dev).roll(i, 0) for i in range(1, nbuf)]
+    outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+    bytes_ = M * 2 * N * 2 + M * N * 2
+
+    ms, ms_kernel = _time_steps(lambda i: silu_and_mul(xs[i % nbuf], outs[i % nbuf]), steps, warmup)
+    res = {
+        "metric": "silu_and_mul HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
+        "ms_per_step": ms, "dtype": "bf16",
+        "config": {"workload": "silu_and_mul bf16 [8192, 2x11008] N(0,1) seed 0"},
+        "roofline": {"kernel": "silu_and_mul_vec16", "bound": "hbm",
+                     "achieved": bytes_ / ms_kernel / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": bytes_ / ms_kernel / 1e6 / PEAK_HBM_GBS,
+                     "traffic": _traffic("silu_and_mul")},
+    }
+    if cpu:
+        from oracle import activation as oa
+
+        rows = 1024
+        sample = x0[:rows]
+        oa.silu_and_mul(sample[:64])
+        t0 = time.perf_counter()
+        reps = 3
+        for _ in range(reps):
+            oa.silu_and_mul(sample)
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": bytes_ * rows / M / dt / 1e9, "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{rows} of {M} rows, {reps} reps"}
+    return res
+
+
+def wl_gating(dev, steps, warmup, cpu):
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size, moe_topk_softmax
+
+    T, E, K, BLK = 16384, 64, 6, 64
+    logits_cpu = torch.randn((T, E), generator=_gen(1))
+    logits = logits_cpu.to(dev)
+
+    def step(i):
+        w, ids = moe_topk_softmax(logits, K)
+        return moe_align_block_size(ids, BLK, E)
+
+    _, _, npad = step(0)
+    l_pad = int(npad.item())
+    bytes_ = (T * E * 4 + T * K * 4 * 2 + T * K * 4 + 4 * l_pad + 4 * l_pad // BLK + E * 4 + 4)
+    ms, _ = _time_steps(step, steps, warmup)
+
+    # the same two calls replayed from a HIP graph (no Python / launch latency in between)
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(0)
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            out = step(0)
+        for _ in range(warmup):
+            g.replay()
+        torch.cuda.synchronize()
+        t = Timer()
+        ev = t.start()
+        for _ in range(steps):
+            g.replay()
+        t.stop(ev)
+        graph_ms = t.mean_ms() / steps
+        del out
+    except Exception as exc:  # graph capture is optional reporting
+        graph_ms = None
+        print(f"[bench] gating graph replay skipped: {exc}", file=sys.stderr)
+
+    # dominant kernel: the router (reads the logits, 72% of the bytes)
+    tk = Timer()
+    for i in range(steps):
+        e = tk.start()
+        moe_topk_softmax(logits, K)
+        tk.stop(e)
+    ms_router = tk.mean_ms()
+    router_bytes = T * E * 4 + T * K * 8
+    res = {
+        "metric": "MoE gating HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
+        "ms_per_step": ms, "dtype": "f32",
+        "config": {"workload": "moe_topk_softmax + moe_align_block_size fp32 [16384, 64] k=6 block 64 seed 1",
+                   "padded_len": l_pad, "algorithmic_bytes": bytes_},
+        "graph_replay": None if graph_ms is None else {
+            "ms_per_step": graph_ms, "value": bytes_ / graph_ms / 1e6, "unit": "GB/s"},
+        "roofline": {"kernel": "moe_topk_softmax_kernel", "bound": "hbm",
+                     "achieved": router_bytes / ms_router / 1e6, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": router_bytes / ms_router / 1e6 / PEAK_HBM_GBS,
+                     "traffic": _traffic("moe_topk_softmax"),
+                     "note": "4 MB working set: launch-latency bound, served from cache"},
+    }
+    if cpu:
+        from oracle import moe_gating as og
+
+        t0 = time.perf_counter()
+        reps = 3
+        for _ in range(reps):
+            w, ids = og.topk_softmax(logits_cpu, K)
+            og.align_block_size(ids, BLK, E)
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": bytes_ / dt / 1e9, "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"full workload, {reps} reps"}
+    return res
+
+
+def wl_prefill(dev, steps, warmup, cpu):
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    g = _gen(2)
+    lens = torch.randint(512, 4097, (8,), generator=g)
+    cu = torch.zeros(9, dtype=torch.int32)
+    cu[1:] = lens.cumsum(0)
+    total = int(cu[-1])
+    q_cpu = torch.randn((total, 32, 128), generator=g).bfloat16()
+    k_cpu = torch.randn((total, 8, 128), generator=g).bfloat16()
+    v_cpu = torch.randn((total, 8, 128), generator=g).bfloat16()
+    q, k, v = q_cpu.to(dev), k_cpu.to(dev), v_cpu.to(dev)
+    o = torch.empty_like(q)
+    start, seqlen = cu[:-1].to(dev), (cu[1:] - cu[:-1]).to(dev)
+    max_len = int(lens.max())
+    flops = 4 * 128 * 32 * sum(int(l) * (int(l) + 1) // 2 for l in lens)
+
+    ms, ms_kernel = _time_steps(
+        lambda i: context_attention_fwd(q, k, v, o, start, seqlen, max_len), steps, warmup)
+    res = {
+        "metric": "prefill attention TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
+        "ms_per_step": ms, "dtype": "bf16",
+        "config": {"workload": "context_attention_fwd causal varlen, 8 seqs U[512,4096] seed 2, "
+                               "32q/8kv heads, d128, bf16", "total_tokens": total,
+                   "algorithmic_flops": flops},
+        "roofline": {"kernel": "prefill_attn_kernel", "bound": "mfma",
+                     "achieved": flops / ms_kernel / 1e9, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / ms_kernel / 1e9 / PEAK_BF16_TFLOPS,
+                     "traffic": _traffic("prefill_attn")},
+    }
+    if cpu:
+        from oracle import attention as oa
+
+        L = 1024  # one 1024-token sequence, all heads
+        qs, ks, vs = q_cpu[:L], k_cpu[:L], v_cpu[:L]
+        t0 = time.perf_counter()
+        oa.prefill_attention(qs, ks, vs, torch.tensor([0]), torch.tensor([L]))
+        dt = time.perf_counter() - t0
+        sflops = 4 * 128 * 32 * L * (L + 1) // 2
+        res["cpu_baseline"] = {"value": sflops / dt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"one {L}-token sequence, 32 heads, 1 rep"}
+    return res
+
+
+def wl_decode(dev, steps, warmup, cpu):
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+
+    g = _gen(3)
+    B, HQ, HKV, D, PAGE = 64, 32, 8, 128, 64
+    ctx = torch.randint(512, 8193, (B,), generator=g)
+    blocks = (ctx + PAGE - 1) // PAGE
+    num_pages = int(blocks.sum())
+    perm = torch.randperm(num_pages, generator=g).to(torch.int32)
+    table = torch.zeros((B, 128), dtype=torch.int32)
+    at = 0
+    for b in range(B):
+        table[b, :blocks[b]] = perm[at:at + blocks[b]]
+        at += int(blocks[b])
+    kc_cpu = torch.randn((num_pages, PAGE, HKV, D), generator=g).bfloat16()
+    vc_cpu = torch.randn((num_pages, PAGE, HKV, D), generator=g).bfloat16()
+    q_cpu = torch.randn((B, HQ, D), generator=g).bfloat16()
+    nbuf = 2  # two cache copies: 2 x 1.1 GB, well past the 256 MB last-level cache
+    kcs = [kc_cpu.to(dev) for _ in range(nbuf)]
+    vcs = [vc_cpu.to(dev) for _ in range(nbuf)]
+    q, o = q_cpu.to(dev), torch.empty((B, HQ, D), dtype=torch.bfloat16, device=dev)
+    table_d, ctx_d = table.to(dev), ctx.to(torch.int32).to(dev)
+    ones = torch.ones(B, dtype=torch.int32, device=dev)
+    sum_ctx = int(ctx.sum())
+    bytes_ = sum_ctx * HKV * D * 2 * 2 + 2 * B * HQ * D * 2 + table.numel() * 4 + B * 4
+    flops = 4 * D * HQ * sum_ctx
+
+    def step(i):
+        paged_attention_fwd(q, kcs[i % nbuf], vcs[i % nbuf], o, table_d, None, ones, ctx_d, 1)
+
+    ms, ms_kernel = _time_steps(step, steps, warmup)
+    res = {
+        "metric": "paged decode attention HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
+        "ms_per_step": ms, "dtype": "bf16", "tflops": flops / ms / 1e9,
+        "config": {"workload": "paged_attention_fwd decode, batch 64, ctx U[512,8192] seed 3, "
+                               "64-token pages, 32q/8kv heads, d128, bf16",
+                   "sum_ctx": sum_ctx, "algorithmic_bytes": bytes_},
+        "roofline": {"kernel": "paged_decode_split_kernel (+combine)", "bound": "hbm",
+                     "achieved": bytes_ / ms_kernel / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": bytes_ / ms_kernel / 1e6 / PEAK_HBM_GBS,
+                     "traffic": _traffic("paged_decode")},
+    }
+    if cpu:
+        from oracle import attention as oa
+
+        n = 8
+        t0 = time.perf_counter()
+        oa.paged_decode(q_cpu[:n], kc_cpu, vc_cpu, table[:n], ctx[:n])
+        dt = time.perf_counter() - t0
+        sbytes = int(ctx[:n].sum()) * HKV * D * 4
+        res["cpu_baseline"] = {"value": sbytes / dt / 1e9, "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {n} of {B} sequences, 1 rep"}
+    return res
+
+
+def wl_moe_fp8(dev, steps, warmup, cpu):
+    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8
+    from oracle import fp8 as ofp8
+    from oracle import moe_gating as og
+
+    T, H, I, E, K = 4096, 2048, 1408, 64, 6
+    g = _gen(5)
+    x_cpu = torch.randn((T, H), generator=g).bfloat16()
+    logits = torch.randn((T, E), generator=g)
+    tw_cpu, ids_cpu = og.topk_softmax(logits, K)   # input preparation, untimed
+    w1q = torch.empty((E, 2 * I, H), dtype=torch.float8_e4m3fn)
+    w1s = torch.empty((E, 2 * I // 128, H // 128))
+    w2q = torch.empty((E, H, I), dtype=torch.float8_e4m3fn)
+    w2s = torch.empty((E, H // 128, I // 128))
+    for e in range(E):  # offline weight quantisation (input preparation, untimed)
+        w1q[e], w1s[e] = ofp8.block_quant_weight(torch.randn((2 * I, H), generator=g) * 0.02)
+        w2q[e], w2s[e] = ofp8.block_quant_weight(torch.randn((H, I), generator=g) * 0.02)
+    x, tw, ids = x_cpu.to(dev), tw_cpu.to(dev), ids_cpu.to(dev)
+    dw = [t.to(dev) for t in (w1q, w1s, w2q, w2s)]
+    flops = 2 * T * K * H * 2 * I + 2 * T * K * I * H
+    gate_up_flops = 2 * T * K * H * 2 * I
+
+    ms, _ = _time_steps(lambda i: fused_moe_fp8(x, *dw, tw, ids, K), steps, warmup)
+
+    stage_t = {}
+    state = {"name": None, "ev": None}
+
+    def hook(name):
+        if state["name"] is not None:
+            stage_t.setdefault(state["name"], Timer()).stop(state["ev"])
+        state["name"] = name
+        if name is not None:
+            state["ev"] = stage_t.setdefault(name, Timer()).start()
+
+    for i in range(steps):
+        fused_moe_fp8(x, *dw, tw, ids, K, _stage_hook=hook)
+    stages = {k: v.mean_ms() for k, v in stage_t.items()}
+    ms_gate_up = stages["gate_up"]
+    res = {
+        "metric": "fp8 fused-MoE TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
+        "ms_per_step": ms, "dtype": "fp8_e4m3",
+        "config": {"workload": "fused_moe_fp8 T=4096 H=2048 I=1408 E=64 top-6, fp8 e4m3 weights "
+                               "128x128 block scales, per-token-group act quant, seed 5",
+                   "algorithmic_flops": flops},
+        "stages_ms": stages,
+        "gemm_only_tflops": flops / (stages["gate_up"] + stages["down"]) / 1e9,
+        "roofline": {"kernel": "moe_gemm_fp8_kernel<gate_up>", "bound": "mfma",
+                     "achieved": gate_up_flops / ms_gate_up / 1e9, "peak": PEAK_FP8_TFLOPS,
+                     "unit": "TFLOP/s", "frac": gate_up_flops / ms_gate_up / 1e9 / PEAK_FP8_TFLOPS,
+                     "traffic": _traffic("moe_gemm_fp8_gate_up")},
+    }
+    if cpu:
+        from oracle import fused_moe as ofm
+
+        n = 64
+        t0 = time.perf_counter()
+        ofm.fused_moe_fp8(x_cpu[:n], w1q, w1s, w2q, w2s, tw_cpu[:n], ids_cpu[:n])
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": flops * n / T / dt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {n} of {T} tokens (all 64 experts de-quantised), 1 rep"}
+    return res
+
+
+WORKLOADS = {
+    "silu_and_mul": wl_silu,
+    "moe_gating": wl_gating,
+    "prefill_attention": wl_prefill,
+    "paged_decode": wl_decode,
+    "moe_fp8": wl_moe_fp8,
+}
+PRIMARY = "moe_fp8"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the operators are single-device; "
+              "no collective is part of the path) -- run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from dlcompiler_amd import _lib
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+    primary = PRIMARY if args.workload == "all" else args.workload
+    results = {}
+    for name in names:
+        t0 = time.perf_counter()
+        results[name] = WORKLOADS[name](dev, args.steps, args.warmup, not args.no_cpu)
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        print(f"[bench] {name}: {results[name]['value']:.2f} {results[name]['unit']} "
+              f"({results[name]['ms_per_step'] * 1e3:.1f} us/step, roofline "
+              f"{results[name]['roofline']['frac'] * 100:.1f}%) in {time.perf_counter() - t0:.1f}s",
+              file=sys.stderr, flush=True)
+    p = results[primary]
+    line = {
+        "metric": p["metric"], "value": p["value"], "unit": p["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": p["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": p["dtype"],
+        "data": "synthetic", "config": p["config"], "roofline": p["roofline"],
+        "cpu_baseline": p.get("cpu_baseline"),
+        "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
+        "workloads": results,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

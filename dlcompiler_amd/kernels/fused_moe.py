@@ -62,7 +62,8 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
                   topk: int,
                   expert_offset: int = 0,
                   num_experts: int = None,
-                  renormalize: bool = False) -> torch.Tensor:
+                  renormalize: bool = False,
+                  _stage_hook=None) -> torch.Tensor:
     """fp8 MoE MLP: per-token-group quant -> gate_up grouped GEMM (+SiLU-and-mul, re-quant)
     -> down grouped GEMM (x routing weight) -> sum over the top-k slots.
 
@@ -71,7 +72,9 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     ``w2_s`` [E, H/128, I/128]); ``topk_weights``/``topk_ids`` [T, topk].  ``E`` is the
     number of local experts, holding global experts ``expert_offset .. expert_offset + E``;
     ``num_experts`` the global count (defaults to ``E``), as in the reference.
+    ``_stage_hook(name)`` is called before each stage (profiling aid).
     """
+    hook = _stage_hook or (lambda name: None)
     _lib.require_cuda(hidden_states, w1_q, w1_s, w2_q, w2_s, topk_weights, topk_ids)
     assert hidden_states.dim() == 2 and topk_ids.shape == topk_weights.shape
     T, H = hidden_states.shape
@@ -94,9 +97,12 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     w1_s = w1_s.to(torch.float32).contiguous()
     w2_s = w2_s.to(torch.float32).contiguous()
 
+    hook("align")
     sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, _ALIGN_BLOCK, num_experts)
     num_mblocks = expert_ids.numel()
+    hook("quant")
     xq, xs = per_token_group_quant_fp8(hidden_states)
+    hook("alloc")
 
     rows = num_mblocks * _ALIGN_BLOCK
     hq = torch.empty((rows, I), dtype=torch.float8_e4m3fn, device=dev)
@@ -108,18 +114,22 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     lib = _lib.load()
     stream = _lib.current_stream_ptr(dev)
     with torch.cuda.device(dev):
+        hook("gate_up")
         st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
                                           w1_s.data_ptr(), sorted_ids.data_ptr(),
                                           expert_ids.data_ptr(), num_mblocks, T, topk, H, I,
                                           expert_offset, E, hq.data_ptr(), hs.data_ptr(), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_gate_up")
+        hook("down")
         st = lib.dlb_moe_gemm_fp8_down(hq.data_ptr(), hs.data_ptr(), w2_q.data_ptr(),
                                        w2_s.data_ptr(), sorted_ids.data_ptr(),
                                        expert_ids.data_ptr(), topk_weights.data_ptr(),
                                        num_mblocks, T, topk, H, I, expert_offset, E,
                                        slots.data_ptr(), _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_down")
+        hook("topk_sum")
         st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), T, topk, H,
                                   _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_topk_sum")
+        hook(None)
     return out
