@@ -82,7 +82,7 @@ struct MoeGemmParams {
   const float* a_scale;       // [rows, K / 128]
   const unsigned char* w;     // weights fp8 [E_local, N, K]
   const float* w_scale;       // [E_local, N / 128, K / 128]
-  const int32_t* sorted_ids;  // [num_mblocks * 64]
+  const int32_t* sorted_ids;  // [num_mblocks * BM]
   const int32_t* expert_ids;  // [num_mblocks]
   int num_mblocks, num_ntiles, grid_real;
   int K, N, KC;               // KC = K / 128
@@ -91,15 +91,14 @@ struct MoeGemmParams {
   int expert_offset;          // weights hold experts [expert_offset, expert_offset + E_local)
   int num_local;              // E_local
   // gate_up flavour
-  unsigned char* hq;          // [num_mblocks * 64, I]
-  float* hs;                  // [num_mblocks * 64, I / 128]
+  unsigned char* hq;          // [num_mblocks * BM, I]
+  float* hs;                  // [num_mblocks * BM, I / 128]
   int I;
   // down flavour
   void* out;                  // [numel, N] bf16/f16
   const float* topk_w;        // [numel]
 };
 
-constexpr int kBM = 64;         // rows (routing slots) per workgroup = alignment block
 constexpr int kARow = 128 + 16; // LDS row pitch of the activation chunk (bytes)
 
 __device__ __forceinline__ f32x4 mfma_fp8(const i32x8& a, const i32x8& b) {
@@ -111,8 +110,13 @@ __device__ __forceinline__ f32x4 mfma_fp8(const i32x8& a, const i32x8& b) {
 // GATED = true : gate_up GEMM (N = 2I), tile = 128 gate cols + the matching 128 up cols,
 //                epilogue silu(gate) * up -> fp8 + per-128 scale, rows kept in sorted order.
 // GATED = false: down GEMM, tile = 256 cols, epilogue * routing weight -> out[slot, n].
-template <bool GATED, int DT>
+// BM = rows (routing slots) per workgroup = the alignment block of the routing (64 or 128).
+template <bool GATED, int DT, int BM>
 __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
+  constexpr int kBM = BM;
+  constexpr int MT = BM / 16;          // 16-token sub-tiles
+  constexpr int TPR = 256 / BM;        // staging threads per activation row
+  constexpr int AU = 8 / TPR;          // 16-byte units per staging thread
   __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][kBM * kARow];
   __shared__ __attribute__((aligned(16))) float as_lds[2][kBM];
   __shared__ float red_lds[4][kBM];
@@ -138,9 +142,10 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
   const int K = p.K, KC = p.KC;
 
   if (tid < kBM) sid_lds[tid] = p.sorted_ids[row0 + tid];
+  static_assert(BM == 64 || BM == 128, "BM");
 
   // ---- activation chunk staging: thread -> (row = tid / 4, 32-byte segment = tid % 4)
-  const int arow = tid >> 2, aseg = tid & 3;
+  const int arow = tid / TPR, aseg = tid % TPR;
   const unsigned char* a_ptr;
   const float* as_ptr;
   {
@@ -151,7 +156,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     } else {
       src_row = row0 + arow;
     }
-    a_ptr = p.a + src_row * K + aseg * 32;
+    a_ptr = p.a + src_row * K + aseg * (16 * AU);
     as_ptr = p.a_scale + src_row * KC;
   }
 
@@ -180,23 +185,26 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     ws_ptr[j] = p.w_scale + ((int64_t)e * (p.N >> 7) + sblk[j]) * KC;
   }
 
-  f32x4 acc[4][4];  // [token sub-tile mt][column sub-tile j]
+  f32x4 acc[MT][4];  // [token sub-tile mt][column sub-tile j]
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  u32x4 areg[2];
+  u32x4 areg[AU];
   float asreg = 0.0f;
   i32x8 breg[2][4];
   float bsreg[2][4];
 
   auto load_a = [&](int kc) {
-    areg[0] = *(const u32x4*)(a_ptr + kc * 128);
-    areg[1] = *(const u32x4*)(a_ptr + kc * 128 + 16);
+#pragma unroll
+    for (int u = 0; u < AU; ++u) areg[u] = *(const u32x4*)(a_ptr + kc * 128 + 16 * u);
     if (aseg == 0) asreg = as_ptr[kc];
   };
   auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
+#ifdef DLB_EXP_NO_BLOAD
+    if (kc > 1) return;
+#endif
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const u32x4 lo = *(const u32x4*)(w_ptr[j] + kc * 128);
@@ -207,14 +215,14 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     }
   };
   auto store_a = [&](int buf) {
-    unsigned char* dst = a_lds[buf] + arow * kARow + aseg * 32;
-    *(u32x4*)(dst) = areg[0];
-    *(u32x4*)(dst + 16) = areg[1];
+    unsigned char* dst = a_lds[buf] + arow * kARow + aseg * (16 * AU);
+#pragma unroll
+    for (int u = 0; u < AU; ++u) *(u32x4*)(dst + 16 * u) = areg[u];
     if (aseg == 0) as_lds[buf][arow] = asreg;
   };
   auto compute = [&](int buf, const i32x8 (&b)[4], const float (&bs)[4]) {
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const unsigned char* src = a_lds[buf] + (16 * mt + c) * kARow + 16 * g;
       const u32x4 lo = *(const u32x4*)(src);
       const u32x4 hi = *(const u32x4*)(src + 64);
@@ -223,9 +231,14 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
       const float as = as_lds[buf][16 * mt + c];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+#ifdef DLB_EXP_NO_FMA
+        acc[mt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], x, acc[mt][j], 0, 0, 0, 0, 0, 0);
+        (void)as;
+#else
         const f32x4 part = mfma_fp8(b[j], x);
         const float sc = as * bs[j];
         acc[mt][j] += part * sc;
+#endif
       }
     }
   };
@@ -255,10 +268,10 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
 
   // ---- epilogues: lane holds token (16*mt + c), columns ncol[j] + 4*g + i
   if (GATED) {
-    float h[4][2][4];
-    float amax[4];
+    float h[MT][2][4];
+    float amax[MT];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       amax[mt] = 0.0f;
 #pragma unroll
       for (int jg = 0; jg < 2; ++jg) {
@@ -278,7 +291,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     __syncthreads();
     const int scol = nt;  // 128-column group index of the intermediate
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int r = 16 * mt + c;
       const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
       const float scale = fmaxf(m, kQuantEps) / kFp8Max;
@@ -294,7 +307,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
   } else {
     __syncthreads();  // sid_lds visible (also true after the main loop's barriers)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
       const int sid = sid_lds[16 * mt + c];
       if (sid < p.numel) {
         const float rw = p.topk_w[sid];
@@ -384,13 +397,14 @@ extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs,
 
 extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q,
                                         const float* w1s, const int32_t* sorted_ids,
-                                        const int32_t* expert_ids, int num_mblocks,
+                                        const int32_t* expert_ids, int num_mblocks, int block_m,
                                         int num_tokens, int topk, int H, int I,
                                         int expert_offset, int num_local_experts, void* hq,
                                         float* hs, void* stream) {
   using namespace dlb;
   const int st = check_gemm_common(xq, xs, w1q, w1s, sorted_ids, expert_ids, num_mblocks, H, I);
   if (st != DLB_OK || num_mblocks == 0) return st;
+  if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
   if (num_tokens < 1 || topk < 1 || num_local_experts < 1 || !hq || !hs) return DLB_ERR_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(hq) & 3u) != 0) return DLB_ERR_UNSUPPORTED;
   MoeGemmParams p = {};
@@ -415,20 +429,26 @@ extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const v
   p.I = I;
   p.grid_real = p.num_mblocks * p.num_ntiles;
   const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
-  hipLaunchKernelGGL((moe_gemm_fp8_kernel<true, DLB_DTYPE_BF16>), dim3(grid), dim3(256), 0,
-                     (hipStream_t)stream, p);
+  if (block_m == 128)
+    hipLaunchKernelGGL((moe_gemm_fp8_kernel<true, DLB_DTYPE_BF16, 128>), dim3(grid), dim3(256), 0,
+                       (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL((moe_gemm_fp8_kernel<true, DLB_DTYPE_BF16, 64>), dim3(grid), dim3(256), 0,
+                       (hipStream_t)stream, p);
   return launch_status();
 }
 
 extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q,
                                      const float* w2s, const int32_t* sorted_ids,
                                      const int32_t* expert_ids, const float* topk_weights,
-                                     int num_mblocks, int num_tokens, int topk, int H, int I,
-                                     int expert_offset, int num_local_experts, void* out,
+                                     int num_mblocks, int block_m, int num_tokens, int topk,
+                                     int H, int I, int expert_offset, int num_local_experts,
+                                     void* out,
                                      int out_dtype, void* stream) {
   using namespace dlb;
   const int st = check_gemm_common(hq, hs, w2q, w2s, sorted_ids, expert_ids, num_mblocks, I, H);
   if (st != DLB_OK || num_mblocks == 0) return st;
+  if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
   if (num_tokens < 1 || topk < 1 || num_local_experts < 1 || !out || !topk_weights)
     return DLB_ERR_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(out) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
@@ -454,14 +474,19 @@ extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void
   p.I = I;
   p.grid_real = p.num_mblocks * p.num_ntiles;
   const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
-  if (out_dtype == DLB_DTYPE_BF16)
-    hipLaunchKernelGGL((moe_gemm_fp8_kernel<false, DLB_DTYPE_BF16>), dim3(grid), dim3(256), 0,
-                       (hipStream_t)stream, p);
-  else if (out_dtype == DLB_DTYPE_F16)
-    hipLaunchKernelGGL((moe_gemm_fp8_kernel<false, DLB_DTYPE_F16>), dim3(grid), dim3(256), 0,
-                       (hipStream_t)stream, p);
-  else
+#define DLB_LAUNCH_DOWN(DT_, BM_)                                                              \
+  hipLaunchKernelGGL((moe_gemm_fp8_kernel<false, DT_, BM_>), dim3(grid), dim3(256), 0,         \
+                     (hipStream_t)stream, p)
+  if (out_dtype == DLB_DTYPE_BF16) {
+    if (block_m == 128) DLB_LAUNCH_DOWN(DLB_DTYPE_BF16, 128);
+    else DLB_LAUNCH_DOWN(DLB_DTYPE_BF16, 64);
+  } else if (out_dtype == DLB_DTYPE_F16) {
+    if (block_m == 128) DLB_LAUNCH_DOWN(DLB_DTYPE_F16, 128);
+    else DLB_LAUNCH_DOWN(DLB_DTYPE_F16, 64);
+  } else {
     return DLB_ERR_UNSUPPORTED;
+  }
+#undef DLB_LAUNCH_DOWN
   return launch_status();
 }
 

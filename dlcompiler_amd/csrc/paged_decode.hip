@@ -18,6 +18,8 @@
 //     registers ARE the B operand of O^T = V^T.P^T: P never moves between lanes.
 // The kernel is an HBM stream (4 FLOP/byte at GQA 4:1); everything else is sized to keep
 // tens of KB of loads in flight per CU.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace dlb {
@@ -76,31 +78,34 @@ struct Mma16<DLB_DTYPE_F16> {
 constexpr int kTile = 64;          // keys per iteration
 constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
 
-template <int DT, int D>
-__global__ __launch_bounds__(64) void paged_decode_split_kernel(const DecodeParams p) {
+// WPB wavefronts per workgroup: wave w handles (kv head, head chunk) unit blockIdx.y * WPB + w
+// of the SAME (sequence, KV chunk), so the waves of a workgroup read neighbouring 256-byte
+// head slices of the same token rows at the same time (whole 2 KB token rows in flight).
+template <int DT, int D, int WPB, bool POW2>
+__global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const DecodeParams p) {
   constexpr int KS = D / 32;   // MFMA k-steps over the head dim
   constexpr int MT = D / 16;   // 16-row tiles of O^T
-  constexpr int VIT = D / 32;  // V staging iterations (64 lanes x 4 keys x 8 dims each)
   constexpr int DG = D / 8;    // 8-dim groups per key row
 
   const int split = blockIdx.x;
-  const int kvh = blockIdx.y / p.hchunks;
-  const int hchunk = blockIdx.y - kvh * p.hchunks;
+  const int wave = threadIdx.x >> 6;
+  const int unit = blockIdx.y * WPB + wave;
+  const int kvh = unit / p.hchunks;
+  const int hchunk = unit - kvh * p.hchunks;
   const int b = blockIdx.z;
   const int ctx = p.kv_len[b];
   const int k_begin = split * p.keys_per_split;
   if (k_begin >= ctx) return;  // uniform for the wave; also covers ctx <= 0
   const int k_end = min(ctx, k_begin + p.keys_per_split);
 
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
   const int g = lane >> 4;  // lane group 0..3
   const int c = lane & 15;  // column (query head) / row (key) inside a 16-tile
 
-  __shared__ __attribute__((aligned(16))) unsigned char vt[D * kVtRowBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char vt_all[WPB][D * kVtRowBytes];
+  unsigned char* vt = vt_all[wave];
 
   const unsigned short* qb = (const unsigned short*)p.q;
-  const unsigned short* kb = (const unsigned short*)p.k;
-  const unsigned short* vb = (const unsigned short*)p.v;
   const int32_t* bt = p.block_table + (int64_t)b * p.bt_stride;
 
   // Q^T as the B operand: lane (n = query head c, k = dims 32*ks + 8g .. +8)
@@ -121,46 +126,50 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(const DecodePara
   float m_run = -__builtin_inff();
   float l_run = 0.0f;  // per-lane partial of the softmax denominator
 
-  auto page_of = [&](int key, int& in_page) -> int64_t {
-    int pi;
-    if (p.page_shift >= 0) {
-      pi = key >> p.page_shift;
-      in_page = key & (p.page - 1);
-    } else {
-      pi = key / p.page;
-      in_page = key - pi * p.page;
-    }
-    return (int64_t)bt[pi];
-  };
+  // Addressing: a 16-key sub-tile never straddles a page (page % 16 == 0), so its physical
+  // page comes from ONE wave-uniform block-table entry (a scalar load) and every lane adds a
+  // 32-bit byte offset to a uniform 64-bit base.
+  const unsigned char* kbytes = (const unsigned char*)p.k + (int64_t)kvh * p.k_sh * 2;
+  const unsigned char* vbytes = (const unsigned char*)p.v + (int64_t)kvh * p.v_sh * 2;
+  const uint32_t k_tok_bytes = (uint32_t)p.k_st * 2u, v_tok_bytes = (uint32_t)p.v_st * 2u;
+  constexpr int VL = 64 / DG < 4 ? 64 / DG : 4;  // 4-key groups of a sub-tile staged per pass
+  constexpr int VPASS = 4 / VL;                  // passes per 16-key sub-tile
+  const int dg = lane % DG, kgl = lane / DG;     // lanes with kgl >= VL idle (D < 128)
 
   for (int t0 = k_begin; t0 < k_end; t0 += kTile) {
     // ---- K tile: 4 sub-tiles of 16 keys, straight into A-operand registers ----
     u32x4 kf[4][KS];
+    u32x4 vr[4][VPASS][4];
 #pragma unroll
     for (int sub = 0; sub < 4; ++sub) {
-      const int key = min(t0 + 16 * sub + c, ctx - 1);  // clamp: never read past the context
-      int in_page;
-      const int64_t pg = page_of(key, in_page);
-      const unsigned short* kp = kb + pg * p.k_sp + (int64_t)in_page * p.k_st + (int64_t)kvh * p.k_sh;
+      const int base_key = min(t0 + 16 * sub, ctx - 1);  // uniform; clamp: never read past ctx
+      const int pi = POW2 ? (base_key >> p.page_shift) : (base_key / p.page);
+      const int64_t pg = (int64_t)bt[pi];
+      const int page_key0 = pi * p.page;
+      {
+        const int key = min(t0 + 16 * sub + c, ctx - 1);
+        const unsigned char* base = kbytes + pg * p.k_sp * 2;
+        // K rows are read as two half-line (64-byte) pieces by consecutive k-steps: keep them
+        // cacheable so the second piece hits the line the first one brought in
+        const uint32_t off = (uint32_t)(key - page_key0) * k_tok_bytes + 16u * g;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) kf[sub][ks] = *(const u32x4*)(kp + 32 * ks + 8 * g);
-    }
-    // ---- V tile: each lane takes 4 consecutive keys x 8 dims per iteration ----
-    u32x4 vr[VIT][4];
+        for (int ks = 0; ks < KS; ++ks) kf[sub][ks] = *(const u32x4*)(base + off + 64 * ks);
+      }
+      // ---- V: each lane takes 4 consecutive keys x 8 dims
+      {
+        const unsigned char* base = vbytes + pg * p.v_sp * 2;
 #pragma unroll
-    for (int it = 0; it < VIT; ++it) {
-      const int u = it * 64 + lane;
-      const int dg = u % DG, kg = u / DG;
-      const int key0 = min(t0 + 4 * kg, ctx - 1);
-      int in_page;
-      const int64_t pg = page_of(key0, in_page);
-      const unsigned short* vp = vb + pg * p.v_sp + (int64_t)kvh * p.v_sh + 8 * dg;
-      // the 4 keys share a page (page % 16 == 0); clamp each inside the context
-      const int room = ctx - 1 - key0;
+        for (int ps = 0; ps < VPASS; ++ps) {
+          const int key0 = min(t0 + 16 * sub + 4 * (ps * VL + kgl), ctx - 1);
+          const int room = ctx - 1 - key0;
+          if (kgl < VL) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int rr = min(r, room);
-        vr[it][r] = *(const u32x4*)(vp + (int64_t)(in_page + rr) * p.v_st);
+            for (int r = 0; r < 4; ++r) {
+              const uint32_t off = (uint32_t)(key0 - page_key0 + min(r, room)) * v_tok_bytes + 16u * dg;
+              vr[sub][ps][r] = __builtin_nontemporal_load((const u32x4*)(base + off));
+            }
+          }
+        }
       }
     }
 
@@ -176,22 +185,27 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(const DecodePara
     // ---- V^T into LDS: Vt[d][pos], pos = 32*s + 8*g' + 4*a + r for key 32*s + 16*a + 4*g' + r
     __syncthreads();  // previous tile's operand reads are done
 #pragma unroll
-    for (int it = 0; it < VIT; ++it) {
-      const int u = it * 64 + lane;
-      const int dg = u % DG, kg = u / DG;
-      const int unit = 4 * (kg >> 3) + (kg & 3);  // 16-byte unit inside the row
-      const int half = (kg >> 2) & 1;             // 8-byte half inside the unit
+    for (int sub = 0; sub < 4; ++sub) {
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const unsigned int lo01 = __builtin_amdgcn_perm(vr[it][1][w], vr[it][0][w], 0x05040100u);
-        const unsigned int lo23 = __builtin_amdgcn_perm(vr[it][3][w], vr[it][2][w], 0x05040100u);
-        const unsigned int hi01 = __builtin_amdgcn_perm(vr[it][1][w], vr[it][0][w], 0x07060302u);
-        const unsigned int hi23 = __builtin_amdgcn_perm(vr[it][3][w], vr[it][2][w], 0x07060302u);
-        const int d0 = 8 * dg + 2 * w;
-        const int sw = ((d0 >> 4) & 3) << 1;  // same for d0 and d0 + 1
-        unsigned char* row = vt + d0 * kVtRowBytes + ((unit ^ sw) << 4) + (half << 3);
-        *(u32x2*)(row) = u32x2{lo01, lo23};
-        *(u32x2*)(row + kVtRowBytes) = u32x2{hi01, hi23};
+      for (int ps = 0; ps < VPASS; ++ps) {
+        if (kgl < VL) {
+          // key group kg = 4 * sub + (ps * VL + kgl) inside the 64-key tile
+          const int unit = 4 * (sub >> 1) + ps * VL + kgl;  // 16-byte unit inside the row
+          const int half = sub & 1;                         // 8-byte half inside the unit
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            const u32x4* v4 = vr[sub][ps];
+            const unsigned int lo01 = __builtin_amdgcn_perm(v4[1][w], v4[0][w], 0x05040100u);
+            const unsigned int lo23 = __builtin_amdgcn_perm(v4[3][w], v4[2][w], 0x05040100u);
+            const unsigned int hi01 = __builtin_amdgcn_perm(v4[1][w], v4[0][w], 0x07060302u);
+            const unsigned int hi23 = __builtin_amdgcn_perm(v4[3][w], v4[2][w], 0x07060302u);
+            const int d0 = 8 * dg + 2 * w;
+            const int sw = ((d0 >> 4) & 3) << 1;  // same for d0 and d0 + 1
+            unsigned char* row = vt + d0 * kVtRowBytes + ((unit ^ sw) << 4) + (half << 3);
+            *(u32x2*)(row) = u32x2{lo01, lo23};
+            *(u32x2*)(row + kVtRowBytes) = u32x2{hi01, hi23};
+          }
+        }
       }
     }
 
@@ -292,8 +306,16 @@ int pick_keys_per_split(int B, int Hkv, int hchunks, int max_ctx) {
   // enough work items to cover the chip several times over, but no smaller than 2 tiles
   const int64_t units = (int64_t)B * Hkv * hchunks;
   int kps = 512;
+  if (const char* env = getenv("DLB_DECODE_KPS")) kps = atoi(env);
   while (kps > 128 && units * ((max_ctx + kps - 1) / kps) < 4096) kps >>= 1;
   return kps;
+}
+
+int pick_waves_per_block(int units) {
+  int wpb = 1;
+  if (const char* env = getenv("DLB_DECODE_WPB")) wpb = atoi(env);
+  while (wpb > 1 && units % wpb != 0) wpb >>= 1;
+  return wpb;
 }
 
 }  // namespace
@@ -329,6 +351,9 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   if (page % 16 != 0) return DLB_ERR_UNSUPPORTED;
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
   if ((int64_t)page * max_blocks > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
+  // per-lane byte offsets inside a page are 32-bit
+  if ((int64_t)page * k_stride_tok * 2 > 0x7fffffff || (int64_t)page * v_stride_tok * 2 > 0x7fffffff)
+    return DLB_ERR_UNSUPPORTED;
   // 128-bit operand loads
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return DLB_ERR_UNSUPPORTED;
   const int64_t strides[] = {q_stride_b,   q_stride_h,    k_stride_page, k_stride_tok,
@@ -374,11 +399,25 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   p.ws_ml = p.ws_o + (size_t)B * Hq * p.nsplit_max * D;
 
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid1((uint32_t)p.nsplit_max, (uint32_t)(Hkv * p.hchunks), (uint32_t)B);
+  const int units = Hkv * p.hchunks;
+  const int wpb = pick_waves_per_block(units);
+  const dim3 grid1((uint32_t)p.nsplit_max, (uint32_t)(units / wpb), (uint32_t)B);
   const dim3 grid2((uint32_t)Hq, (uint32_t)B);
+#define DLB_LAUNCH_DECODE_W(DT_, D_, W_)                                                       \
+  do {                                                                                         \
+    if (p.page_shift >= 0)                                                                     \
+      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, W_, true>), grid1, dim3(64 * W_), \
+                         0, s, p);                                                             \
+    else                                                                                       \
+      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, W_, false>), grid1,               \
+                         dim3(64 * W_), 0, s, p);                                              \
+  } while (0)
 #define DLB_LAUNCH_DECODE(DT_, D_)                                                              \
   do {                                                                                          \
-    hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_>), grid1, dim3(64), 0, s, p);         \
+    if (wpb == 8) DLB_LAUNCH_DECODE_W(DT_, D_, 8);                                              \
+    else if (wpb == 4) DLB_LAUNCH_DECODE_W(DT_, D_, 4);                                         \
+    else if (wpb == 2) DLB_LAUNCH_DECODE_W(DT_, D_, 2);                                         \
+    else DLB_LAUNCH_DECODE_W(DT_, D_, 1);                                                       \
     hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p);       \
   } while (0)
   if (dtype == DLB_DTYPE_BF16) {
@@ -388,6 +427,7 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
     if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
     else DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 64);
   }
+#undef DLB_LAUNCH_DECODE_W
 #undef DLB_LAUNCH_DECODE
   return launch_status();
 }

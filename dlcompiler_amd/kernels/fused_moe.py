@@ -12,7 +12,7 @@ import torch
 from .. import _lib
 from .moe_gating import moe_align_block_size
 
-_ALIGN_BLOCK = 64  # rows per grouped-GEMM workgroup
+_ALIGN_BLOCK = int(__import__('os').environ.get('DLB_MOE_BLOCK', '128'))  # rows per grouped-GEMM workgroup tile
 
 
 def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
@@ -117,14 +117,15 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
         hook("gate_up")
         st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
                                           w1_s.data_ptr(), sorted_ids.data_ptr(),
-                                          expert_ids.data_ptr(), num_mblocks, T, topk, H, I,
-                                          expert_offset, E, hq.data_ptr(), hs.data_ptr(), stream)
+                                          expert_ids.data_ptr(), num_mblocks, _ALIGN_BLOCK, T, topk,
+                                          H, I, expert_offset, E, hq.data_ptr(), hs.data_ptr(),
+                                          stream)
         _lib.check(st, "dlb_moe_gemm_fp8_gate_up")
         hook("down")
         st = lib.dlb_moe_gemm_fp8_down(hq.data_ptr(), hs.data_ptr(), w2_q.data_ptr(),
                                        w2_s.data_ptr(), sorted_ids.data_ptr(),
                                        expert_ids.data_ptr(), topk_weights.data_ptr(),
-                                       num_mblocks, T, topk, H, I, expert_offset, E,
+                                       num_mblocks, _ALIGN_BLOCK, T, topk, H, I, expert_offset, E,
                                        slots.data_ptr(), _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_down")
         hook("topk_sum")

@@ -155,16 +155,17 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
 /* gate_up grouped GEMM + SiLU-and-mul + re-quantisation.
  *   xq [num_tokens, H] fp8, xs [num_tokens, H/128]
  *   w1q [num_local_experts, 2I, H] fp8 (gate rows first), w1s [num_local_experts, 2I/128, H/128]
- *   sorted_ids [num_mblocks * 64], expert_ids [num_mblocks]: output of
- *     dlb_moe_align_block_size with block = 64 (flat slot = token * topk + j, sentinel
+ *   sorted_ids [num_mblocks * block_m], expert_ids [num_mblocks]: output of
+ *     dlb_moe_align_block_size with block = block_m, block_m in {64, 128} = rows per
+ *     workgroup tile (flat slot = token * topk + j, sentinel
  *     num_tokens * topk, expert -1 for unused blocks); blocks whose expert lies outside
  *     [expert_offset, expert_offset + num_local_experts) are skipped
- *   hq [num_mblocks * 64, I] fp8 and hs [num_mblocks * 64, I/128]: row r holds
+ *   hq [num_mblocks * block_m, I] fp8 and hs [num_mblocks * block_m, I/128]: row r holds
  *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r
  * H % 128 == 0, I % 128 == 0. */
 int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q, const float* w1s,
                              const int32_t* sorted_ids, const int32_t* expert_ids,
-                             int num_mblocks, int num_tokens, int topk, int H, int I,
+                             int num_mblocks, int block_m, int num_tokens, int topk, int H, int I,
                              int expert_offset, int num_local_experts, void* hq, float* hs,
                              void* stream);
 
@@ -173,9 +174,9 @@ int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q, c
  * w2q [num_local_experts, H, I] fp8, w2s [num_local_experts, H/128, I/128]. */
 int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q, const float* w2s,
                           const int32_t* sorted_ids, const int32_t* expert_ids,
-                          const float* topk_weights, int num_mblocks, int num_tokens, int topk,
-                          int H, int I, int expert_offset, int num_local_experts, void* out,
-                          int out_dtype, void* stream);
+                          const float* topk_weights, int num_mblocks, int block_m,
+                          int num_tokens, int topk, int H, int I, int expert_offset,
+                          int num_local_experts, void* out, int out_dtype, void* stream);
 
 /* out[t, :] = sum_j in[t * topk + j, :] (fp32 accumulation in slot order, one rounding);
  * replaces intermediate_cache2.sum(dim=1), kernels/fused_moe.py:375.  N % 8 == 0. */
