@@ -309,7 +309,7 @@ def wl_decode(dev, steps, warmup, cpu):
 
 
 def wl_moe_fp8(dev, steps, warmup, cpu):
-    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8
+    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8, shuffle_moe_weight_fp8
     from oracle import fp8 as ofp8
     from oracle import moe_gating as og
 
@@ -327,10 +327,16 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         w2q[e], w2s[e] = ofp8.block_quant_weight(torch.randn((H, I), generator=g) * 0.02)
     x, tw, ids = x_cpu.to(dev), tw_cpu.to(dev), ids_cpu.to(dev)
     dw = [t.to(dev) for t in (w1q, w1s, w2q, w2s)]
+    # weights are re-arranged once at load time into MFMA-operand order (untimed, like the
+    # offline quantisation); DLB_BENCH_PLAIN_WEIGHTS=1 times the row-major layout instead
+    shuffled = os.environ.get("DLB_BENCH_PLAIN_WEIGHTS", "0") != "1"
+    if shuffled:
+        dw[0], dw[2] = shuffle_moe_weight_fp8(dw[0]), shuffle_moe_weight_fp8(dw[2])
     flops = 2 * T * K * H * 2 * I + 2 * T * K * I * H
     gate_up_flops = 2 * T * K * H * 2 * I
 
-    ms, _ = _time_steps(lambda i: fused_moe_fp8(x, *dw, tw, ids, K), steps, warmup)
+    ms, _ = _time_steps(lambda i: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled),
+                        steps, warmup)
 
     stage_t = {}
     state = {"name": None, "ev": None}
@@ -343,7 +349,7 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
             state["ev"] = stage_t.setdefault(name, Timer()).start()
 
     for i in range(steps):
-        fused_moe_fp8(x, *dw, tw, ids, K, _stage_hook=hook)
+        fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled, _stage_hook=hook)
     stages = {k: v.mean_ms() for k, v in stage_t.items()}
     ms_gate_up = stages["gate_up"]
     res = {
@@ -351,6 +357,7 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         "ms_per_step": ms, "dtype": "fp8_e4m3",
         "config": {"workload": "fused_moe_fp8 T=4096 H=2048 I=1408 E=64 top-6, fp8 e4m3 weights "
                                "128x128 block scales, per-token-group act quant, seed 5",
+                   "weight_layout": "operand-order" if shuffled else "row-major",
                    "algorithmic_flops": flops},
         "stages_ms": stages,
         "gemm_only_tflops": flops / (stages["gate_up"] + stages["down"]) / 1e9,

@@ -21,6 +21,8 @@
 // and the epilogues store 4 adjacent outputs.  Weight fragments go straight from HBM/L2 into
 // operand registers (each wave owns its own n range, so nothing is shared between waves);
 // only the 64 x 128-byte activation chunk is staged through LDS, double-buffered.
+#include <type_traits>
+
 #include "common.h"
 
 namespace dlb {
@@ -90,6 +92,7 @@ struct MoeGemmParams {
   int num_tokens;
   int expert_offset;          // weights hold experts [expert_offset, expert_offset + E_local)
   int num_local;              // E_local
+  int w_layout;               // 0: [E, N, K] row-major, 1: MFMA-operand order (see header)
   // gate_up flavour
   unsigned char* hq;          // [num_mblocks * BM, I]
   float* hs;                  // [num_mblocks * BM, I / 128]
@@ -99,7 +102,6 @@ struct MoeGemmParams {
   const float* topk_w;        // [numel]
 };
 
-constexpr int kARow = 128 + 16; // LDS row pitch of the activation chunk (bytes)
 
 __device__ __forceinline__ f32x4 mfma_fp8(const i32x8& a, const i32x8& b) {
   const f32x4 z = {0.f, 0.f, 0.f, 0.f};
@@ -115,10 +117,17 @@ template <bool GATED, int DT, int BM>
 __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
   constexpr int kBM = BM;
   constexpr int MT = BM / 16;          // 16-token sub-tiles
+  constexpr int SKC = 2;               // 128-byte K chunks per activation stage
+#ifndef DLB_MOE_PD
+#define DLB_MOE_PD 2
+#endif
+  constexpr int PD = DLB_MOE_PD;       // weight-fragment ring depth (chunks in flight + 1)
   constexpr int TPR = 256 / BM;        // staging threads per activation row
-  constexpr int AU = 8 / TPR;          // 16-byte units per staging thread
+  constexpr int AU = SKC * 8 / TPR;    // 16-byte units per staging thread and stage
+  constexpr int kARow = SKC * 128 + 16;  // LDS row pitch of an activation stage (bytes)
+  static_assert(SKC <= TPR, "one staging thread per (row, chunk) loads the scale");
   __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][kBM * kARow];
-  __shared__ __attribute__((aligned(16))) float as_lds[2][kBM];
+  __shared__ __attribute__((aligned(16))) float as_lds[2][SKC][kBM];
   __shared__ float red_lds[4][kBM];
   __shared__ int32_t sid_lds[kBM];
 
@@ -156,7 +165,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     } else {
       src_row = row0 + arow;
     }
-    a_ptr = p.a + src_row * K + aseg * (16 * AU);
+    a_ptr = p.a + src_row * K;
     as_ptr = p.a_scale + src_row * KC;
   }
 
@@ -174,14 +183,28 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
 #pragma unroll
     for (int j = 0; j < 4; ++j) ncol[j] = n0 + 16 * j;
   }
-  const unsigned char* w_ptr[4];
+  // Weight addressing: one wave-uniform base per expert (kept in scalar registers) plus a
+  // 32-bit per-lane byte offset per sub-tile; the block scales of a sub-tile are wave-uniform
+  // and come through scalar loads.
+  const unsigned char* wbase = p.w + (int64_t)e * p.N * K;
+  uint32_t woff[4];
   const float* ws_ptr[4];
+  // byte distance between consecutive K chunks / between the two 16-byte operand halves
+  const int w_kc_stride = p.w_layout ? 2048 : 128;
+  const int w_hi_off = p.w_layout ? 1024 : 64;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    sblk[j] = min(ncol[j] >> 7, (p.N >> 7) - 1);
-    // lanes of group g take K bytes [16g, 16g+16) and [64+16g, 64+16g+16) of each chunk
-    const int n = min(ncol[j] + c, p.N - 1);
-    w_ptr[j] = p.w + ((int64_t)e * p.N + n) * K + 16 * g;
+    sblk[j] = __builtin_amdgcn_readfirstlane(min(ncol[j] >> 7, (p.N >> 7) - 1));
+    if (p.w_layout) {
+      // operand-order storage: per (16-row tile, chunk) one 2 KB block = [half][lane][16 B],
+      // so each of the two loads of a fragment is one contiguous 1 KB wave access
+      const int nb = min(ncol[j] >> 4, (p.N >> 4) - 1);
+      woff[j] = (uint32_t)nb * (uint32_t)KC * 2048u + (uint32_t)lane * 16u;
+    } else {
+      // row-major storage: lanes of group g take K bytes [16g, 16g+16) and [64+16g, 64+16g+16)
+      const int n = min(ncol[j] + c, p.N - 1);
+      woff[j] = (uint32_t)n * (uint32_t)K + 16u * g;
+    }
     ws_ptr[j] = p.w_scale + ((int64_t)e * (p.N >> 7) + sblk[j]) * KC;
   }
 
@@ -191,80 +214,124 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Pipeline: activations move global -> registers -> LDS in stages of SKC chunks, one stage
+  // ahead, one barrier per stage; weight fragments sit in a ring of PD chunks, loaded PD-1
+  // chunks ahead of their use; the scale-and-accumulate FMAs of one 16-token step are issued
+  // between the MFMAs of the next step so the matrix pipe does not wait for the VALU.
   u32x4 areg[AU];
   float asreg = 0.0f;
-  i32x8 breg[2][4];
-  float bsreg[2][4];
+  i32x8 breg[PD][4];
+  float bsreg[PD][4];
+  const int NS = (KC + SKC - 1) / SKC;
 
-  auto load_a = [&](int kc) {
+  auto load_a = [&](int st) {  // stage st -> registers (chunks past K are clamped, unused)
+    const int kc0 = st * SKC;
 #pragma unroll
-    for (int u = 0; u < AU; ++u) areg[u] = *(const u32x4*)(a_ptr + kc * 128 + 16 * u);
-    if (aseg == 0) asreg = as_ptr[kc];
-  };
-  auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
-#ifdef DLB_EXP_NO_BLOAD
-    if (kc > 1) return;
-#endif
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const u32x4 lo = *(const u32x4*)(w_ptr[j] + kc * 128);
-      const u32x4 hi = *(const u32x4*)(w_ptr[j] + kc * 128 + 64);
-      b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
-                   (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-      bs[j] = ws_ptr[j][kc];
+    for (int u = 0; u < AU; ++u) {
+      const int byte = aseg * (16 * AU) + 16 * u;  // inside the stage's SKC * 128 bytes
+      const int kc = min(kc0 + (byte >> 7), KC - 1);
+      areg[u] = *(const u32x4*)(a_ptr + kc * 128 + (byte & 127));
     }
+    if (aseg < SKC) asreg = as_ptr[min(kc0 + aseg, KC - 1)];
   };
   auto store_a = [&](int buf) {
     unsigned char* dst = a_lds[buf] + arow * kARow + aseg * (16 * AU);
 #pragma unroll
     for (int u = 0; u < AU; ++u) *(u32x4*)(dst + 16 * u) = areg[u];
-    if (aseg == 0) as_lds[buf][arow] = asreg;
+    if (aseg < SKC) as_lds[buf][aseg][arow] = asreg;
   };
-  auto compute = [&](int buf, const i32x8 (&b)[4], const float (&bs)[4]) {
+  auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
+    if (kc >= KC) return;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const unsigned char* src = a_lds[buf] + (16 * mt + c) * kARow + 16 * g;
-      const u32x4 lo = *(const u32x4*)(src);
-      const u32x4 hi = *(const u32x4*)(src + 64);
-      const i32x8 x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
-                            (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-      const float as = as_lds[buf][16 * mt + c];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#ifdef DLB_EXP_NO_FMA
-        acc[mt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j], x, acc[mt][j], 0, 0, 0, 0, 0, 0);
-        (void)as;
-#else
-        const f32x4 part = mfma_fp8(b[j], x);
-        const float sc = as * bs[j];
-        acc[mt][j] += part * sc;
-#endif
-      }
+    for (int j = 0; j < 4; ++j) {
+      const unsigned char* src = wbase + kc * w_kc_stride;
+      const u32x4 lo = *(const u32x4*)(src + woff[j]);
+      const u32x4 hi = *(const u32x4*)(src + w_hi_off + woff[j]);
+      b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+                   (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      bs[j] = ws_ptr[j][kc];
     }
   };
 
-  load_a(0);
-  load_b(0, breg[0], bsreg[0]);
-  for (int kc = 0; kc < KC; kc += 2) {
-    // even chunk: buffers 0
-    store_a(0);
-    __syncthreads();
-    if (kc + 1 < KC) {
-      load_a(kc + 1);
-      load_b(kc + 1, breg[1], bsreg[1]);
-    }
-    compute(0, breg[0], bsreg[0]);
-    if (kc + 1 < KC) {
-      // odd chunk: buffers 1
-      store_a(1);
-      __syncthreads();
-      if (kc + 2 < KC) {
-        load_a(kc + 2);
-        load_b(kc + 2, breg[0], bsreg[0]);
-      }
-      compute(1, breg[1], bsreg[1]);
-    }
+  // software pipeline state: products of the previous 16-token step and their scales
+  f32x4 pp[4];
+  float psc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    pp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    psc[j] = 0.0f;
   }
+  // A stage is SKC * MT steps of 16 tokens x one chunk.  Step t issues its 4 MFMAs, each
+  // followed by the FMAs that retire one product of step t - 1 (for the first step of a
+  // stage: the last step of the previous stage); the activation fragment of step t + 1 is
+  // fetched from LDS before the MFMAs of step t so its latency hides behind them.
+  auto read_x = [&](int buf, int ci, int mt, i32x8& x, float& as) {
+    const unsigned char* src = a_lds[buf] + (16 * mt + c) * kARow + ci * 128 + 16 * g;
+    const u32x4 lo = *(const u32x4*)(src);
+    const u32x4 hi = *(const u32x4*)(src + 64);
+    x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+              (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    as = as_lds[buf][ci][16 * mt + c];
+  };
+  auto do_stage = [&](auto jtag, int st) {
+    constexpr int J = decltype(jtag)::value;  // st % PD
+    const int buf = st & 1;
+    const int nchunks = min(SKC, KC - st * SKC);  // chunks of this stage that exist (uniform)
+    i32x8 xq[2];
+    float asq[2];
+    read_x(buf, 0, 0, xq[0], asq[0]);
+#pragma unroll
+    for (int ci = 0; ci < SKC; ++ci) {
+      // ring slot of chunk kc = st * SKC + ci is kc % PD, the slot being refilled holds
+      // chunk kc + PD - 1; both are compile-time constants after unrolling
+      constexpr int kBase = (J * SKC) % PD;
+      const int slot = (kBase + ci) % PD;
+      const int refill = (kBase + ci + PD - 1) % PD;
+      if (ci < nchunks) {
+        load_b(st * SKC + ci + PD - 1, breg[refill], bsreg[refill]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int t = ci * MT + mt;
+          const int pm = (mt == 0) ? MT - 1 : mt - 1;
+          // prefetch the next step's fragment (same stage only)
+          if (mt + 1 < MT) {
+            read_x(buf, ci, mt + 1, xq[(t + 1) & 1], asq[(t + 1) & 1]);
+          } else if (ci + 1 < SKC) {
+            if (ci + 1 < nchunks) read_x(buf, ci + 1, 0, xq[(t + 1) & 1], asq[(t + 1) & 1]);
+          }
+          f32x4 pc[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            pc[j] = mfma_fp8(breg[slot][j], xq[t & 1]);
+            acc[pm][j] += pp[j] * psc[j];
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            pp[j] = pc[j];
+            psc[j] = asq[t & 1] * bsreg[slot][j];
+          }
+        }
+      }
+    }
+    if (st + 1 < NS) store_a(buf ^ 1);   // stage st + 1 was loaded into registers a stage ago
+    if (st + 2 < NS) load_a(st + 2);
+    __syncthreads();
+  };
+
+  load_a(0);
+#pragma unroll
+  for (int t = 0; t < PD - 1; ++t) load_b(t, breg[t], bsreg[t]);
+  store_a(0);
+  if (NS > 1) load_a(1);
+  __syncthreads();
+  for (int st = 0; st < NS; st += PD) {
+    do_stage(std::integral_constant<int, 0>{}, st);
+    if (PD > 1 && st + 1 < NS) do_stage(std::integral_constant<int, 1 % PD>{}, st + 1);
+    if (PD > 2 && st + 2 < NS) do_stage(std::integral_constant<int, 2 % PD>{}, st + 2);
+  }
+  // retire the products of the very last step
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[j];
 
   // ---- epilogues: lane holds token (16*mt + c), columns ncol[j] + 4*g + i
   if (GATED) {
@@ -361,6 +428,7 @@ int check_gemm_common(const void* a, const void* a_scale, const void* w, const v
   if (num_mblocks == 0) return DLB_OK;
   if (!a || !a_scale || !w || !w_scale || !sorted_ids || !expert_ids) return DLB_ERR_BAD_ARG;
   if (K % 128 != 0 || N % 128 != 0) return DLB_ERR_UNSUPPORTED;
+  if ((int64_t)N * K >= (int64_t)0xffffffffu) return DLB_ERR_UNSUPPORTED;  // 32-bit lane offsets
   if (!aligned16(a) || !aligned16(w)) return DLB_ERR_UNSUPPORTED;
   return DLB_OK;
 }
@@ -399,8 +467,8 @@ extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const v
                                         const float* w1s, const int32_t* sorted_ids,
                                         const int32_t* expert_ids, int num_mblocks, int block_m,
                                         int num_tokens, int topk, int H, int I,
-                                        int expert_offset, int num_local_experts, void* hq,
-                                        float* hs, void* stream) {
+                                        int expert_offset, int num_local_experts, int w_layout,
+                                        void* hq, float* hs, void* stream) {
   using namespace dlb;
   const int st = check_gemm_common(xq, xs, w1q, w1s, sorted_ids, expert_ids, num_mblocks, H, I);
   if (st != DLB_OK || num_mblocks == 0) return st;
@@ -424,6 +492,7 @@ extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const v
   p.num_tokens = num_tokens;
   p.expert_offset = expert_offset;
   p.num_local = num_local_experts;
+  p.w_layout = w_layout ? 1 : 0;
   p.hq = (unsigned char*)hq;
   p.hs = hs;
   p.I = I;
@@ -443,7 +512,7 @@ extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void
                                      const int32_t* expert_ids, const float* topk_weights,
                                      int num_mblocks, int block_m, int num_tokens, int topk,
                                      int H, int I, int expert_offset, int num_local_experts,
-                                     void* out,
+                                     int w_layout, void* out,
                                      int out_dtype, void* stream) {
   using namespace dlb;
   const int st = check_gemm_common(hq, hs, w2q, w2s, sorted_ids, expert_ids, num_mblocks, I, H);
@@ -469,6 +538,7 @@ extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void
   p.num_tokens = num_tokens;
   p.expert_offset = expert_offset;
   p.num_local = num_local_experts;
+  p.w_layout = w_layout ? 1 : 0;
   p.out = out;
   p.topk_w = topk_weights;
   p.I = I;

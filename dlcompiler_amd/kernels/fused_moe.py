@@ -42,6 +42,18 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
     return xq, xs
 
 
+def shuffle_moe_weight_fp8(w_q: torch.Tensor) -> torch.Tensor:
+    """Re-arrange fp8 expert weights ``[E, N, K]`` into MFMA-operand order (done once, when the
+    weights are loaded): per expert, 16-row tile and 128-byte K chunk one 2 KB block laid out
+    ``[half][lane][16 bytes]`` with ``lane = 16 * (k_piece) + row``, so every operand fetch of
+    the grouped GEMM is a contiguous 1 KB access.  Same bytes and the same block scales."""
+    E, N, K = w_q.shape
+    assert w_q.dtype == torch.float8_e4m3fn and N % 16 == 0 and K % 128 == 0
+    b = w_q.contiguous().view(torch.uint8).view(E, N // 16, 16, K // 128, 2, 4, 16)
+    # (e, nb, row c, kc, half h, piece g, byte) -> (e, nb, kc, h, g, c, byte)
+    return b.permute(0, 1, 3, 4, 5, 2, 6).contiguous().view(E, N, K).view(torch.float8_e4m3fn)
+
+
 def get_start_end(topk_idx: torch.Tensor, sorted_idx: torch.Tensor, num_experts: int):
     """``(exp_start, exp_end)`` of each expert's run in the expert-sorted slot list
     (reference: fused_moe.py:267-293; ``end = cumsum(counts)``, ``start = end - counts``).
@@ -63,6 +75,7 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
                   expert_offset: int = 0,
                   num_experts: int = None,
                   renormalize: bool = False,
+                  weights_shuffled: bool = False,
                   _stage_hook=None) -> torch.Tensor:
     """fp8 MoE MLP: per-token-group quant -> gate_up grouped GEMM (+SiLU-and-mul, re-quant)
     -> down grouped GEMM (x routing weight) -> sum over the top-k slots.
@@ -72,6 +85,8 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     ``w2_s`` [E, H/128, I/128]); ``topk_weights``/``topk_ids`` [T, topk].  ``E`` is the
     number of local experts, holding global experts ``expert_offset .. expert_offset + E``;
     ``num_experts`` the global count (defaults to ``E``), as in the reference.
+    ``weights_shuffled=True`` says ``w1_q``/``w2_q`` went through
+    :func:`shuffle_moe_weight_fp8` (same shapes, operand-order bytes) -- the fast path.
     ``_stage_hook(name)`` is called before each stage (profiling aid).
     """
     hook = _stage_hook or (lambda name: None)
@@ -118,14 +133,15 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
         st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
                                           w1_s.data_ptr(), sorted_ids.data_ptr(),
                                           expert_ids.data_ptr(), num_mblocks, _ALIGN_BLOCK, T, topk,
-                                          H, I, expert_offset, E, hq.data_ptr(), hs.data_ptr(),
-                                          stream)
+                                          H, I, expert_offset, E, int(weights_shuffled),
+                                          hq.data_ptr(), hs.data_ptr(), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_gate_up")
         hook("down")
         st = lib.dlb_moe_gemm_fp8_down(hq.data_ptr(), hs.data_ptr(), w2_q.data_ptr(),
                                        w2_s.data_ptr(), sorted_ids.data_ptr(),
                                        expert_ids.data_ptr(), topk_weights.data_ptr(),
                                        num_mblocks, _ALIGN_BLOCK, T, topk, H, I, expert_offset, E,
+                                       int(weights_shuffled),
                                        slots.data_ptr(), _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_down")
         hook("topk_sum")

@@ -162,12 +162,19 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
  *     [expert_offset, expert_offset + num_local_experts) are skipped
  *   hq [num_mblocks * block_m, I] fp8 and hs [num_mblocks * block_m, I/128]: row r holds
  *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r
- * H % 128 == 0, I % 128 == 0. */
+ * H % 128 == 0, I % 128 == 0.
+ * w_layout selects how the fp8 weight bytes of both GEMMs are stored:
+ *   0  row-major [E, N, K] (the reference's w1/w2 layout);
+ *   1  MFMA-operand order, a one-time re-arrangement done when the weights are loaded: for
+ *      expert e, 16-row tile nb and 128-byte K chunk kc, a 2 KB block at
+ *      ((e * N/16 + nb) * K/128 + kc) * 2048 holding [half h][lane l][16 bytes] =
+ *      W[e][16 nb + l % 16][128 kc + 64 h + 16 (l / 16) .. + 16].  Same bytes, same scales;
+ *      every operand load becomes one contiguous 1 KB access. */
 int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q, const float* w1s,
                              const int32_t* sorted_ids, const int32_t* expert_ids,
                              int num_mblocks, int block_m, int num_tokens, int topk, int H, int I,
-                             int expert_offset, int num_local_experts, void* hq, float* hs,
-                             void* stream);
+                             int expert_offset, int num_local_experts, int w_layout, void* hq,
+                             float* hs, void* stream);
 
 /* down grouped GEMM: out[slot, :] = (h_r W_down^T) * topk_weights[slot] for every real slot
  * (pad rows are skipped), out [num_tokens * topk, H] bf16/f16;
@@ -176,7 +183,8 @@ int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q, cons
                           const int32_t* sorted_ids, const int32_t* expert_ids,
                           const float* topk_weights, int num_mblocks, int block_m,
                           int num_tokens, int topk, int H, int I, int expert_offset,
-                          int num_local_experts, void* out, int out_dtype, void* stream);
+                          int num_local_experts, int w_layout, void* out, int out_dtype,
+                          void* stream);
 
 /* out[t, :] = sum_j in[t * topk + j, :] (fp32 accumulation in slot order, one rounding);
  * replaces intermediate_cache2.sum(dim=1), kernels/fused_moe.py:375.  N % 8 == 0. */

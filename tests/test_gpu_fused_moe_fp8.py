@@ -54,7 +54,7 @@ def _check(out, ref):
                                        (64, 128, 128, 2, 1)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_moe_fp8_parity(dev, T, H, I, E, k, dtype):
-    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8
+    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8, shuffle_moe_weight_fp8
 
     x, w1q, w1s, w2q, w2s, tw, ids = _inputs(T, H, I, E, k, 1, dtype)
     out = fused_moe_fp8(x.to(dev), w1q.to(dev), w1s.to(dev), w2q.to(dev), w2s.to(dev),
@@ -62,6 +62,25 @@ def test_fused_moe_fp8_parity(dev, T, H, I, E, k, dtype):
     ref = ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids)
     assert out.shape == (T, H) and out.dtype == dtype
     _check(out.cpu(), ref)
+    # operand-order weight storage: same bytes re-arranged, so the result is bit-identical
+    out2 = fused_moe_fp8(x.to(dev), shuffle_moe_weight_fp8(w1q.to(dev)), w1s.to(dev),
+                         shuffle_moe_weight_fp8(w2q.to(dev)), w2s.to(dev), tw.to(dev), ids.to(dev),
+                         k, weights_shuffled=True)
+    assert torch.equal(out2, out)
+
+
+def test_weight_shuffle_layout(dev):
+    # the documented address formula of the operand-order layout, checked element by element
+    from dlcompiler_amd.kernels.fused_moe import shuffle_moe_weight_fp8
+
+    E, N, K = 2, 32, 256
+    w = torch.arange(E * N * K, dtype=torch.int64).remainder(251).to(torch.uint8)
+    w = w.view(E, N, K)
+    sh = shuffle_moe_weight_fp8(w.view(torch.float8_e4m3fn).to(dev)).cpu().view(torch.uint8).flatten()
+    for e, nb, kc, h, l, b in [(0, 0, 0, 0, 0, 0), (1, 1, 1, 1, 63, 15), (0, 1, 0, 1, 17, 3),
+                               (1, 0, 1, 0, 40, 9)]:
+        addr = ((e * (N // 16) + nb) * (K // 128) + kc) * 2048 + h * 1024 + l * 16 + b
+        assert sh[addr] == w[e, 16 * nb + l % 16, 128 * kc + 64 * h + 16 * (l // 16) + b]
 
 
 def test_one_hot_routing_reduces_to_a_single_expert_mlp(dev):
@@ -138,8 +157,11 @@ def test_config5_full(dev):
     for e in range(E):                               # quantise expert by expert (memory)
         w1q[e], w1s[e] = ofp8.block_quant_weight(torch.randn((2 * I, H), generator=g) * 0.02)
         w2q[e], w2s[e] = ofp8.block_quant_weight(torch.randn((H, I), generator=g) * 0.02)
-    out = fused_moe_fp8(x.to(dev), w1q.to(dev), w1s.to(dev), w2q.to(dev), w2s.to(dev),
-                        tw.to(dev), ids.to(dev), k).cpu()
+    from dlcompiler_amd.kernels.fused_moe import shuffle_moe_weight_fp8
+
+    out = fused_moe_fp8(x.to(dev), shuffle_moe_weight_fp8(w1q.to(dev)), w1s.to(dev),
+                        shuffle_moe_weight_fp8(w2q.to(dev)), w2s.to(dev), tw.to(dev), ids.to(dev),
+                        k, weights_shuffled=True).cpu()
     assert torch.isfinite(out.float()).all()
     # oracle on a token sample: tokens are independent given the weights
     pick = torch.arange(0, T, 37)
