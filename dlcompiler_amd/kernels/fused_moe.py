@@ -12,7 +12,7 @@ import torch
 from .. import _lib
 from .moe_gating import moe_align_block_size
 
-_ALIGN_BLOCK = int(__import__('os').environ.get('DLB_MOE_BLOCK', '128'))  # rows per grouped-GEMM workgroup tile
+_ALIGN_BLOCK = int(__import__('os').environ.get('DLB_MOE_BLOCK', '64'))  # rows per grouped-GEMM workgroup tile
 
 
 def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
