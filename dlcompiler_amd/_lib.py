@@ -37,6 +37,8 @@ SIGNATURES = {
                                               c_int64, c_int64, c_int64, c_int, c_void_p]),
     "dlb_moe_gemm_fp8_gate_up": (c_int, [c_void_p] * 6 + [c_int] * 9 + [c_void_p] * 3),
     "dlb_moe_gemm_fp8_down": (c_int, [c_void_p] * 7 + [c_int] * 9 + [c_void_p, c_int, c_void_p]),
+    "dlb_moe_gemm_16bit_gate_up": (c_int, [c_void_p] * 4 + [c_int] * 9 + [c_void_p, c_int, c_void_p]),
+    "dlb_moe_gemm_16bit_down": (c_int, [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_int, c_void_p]),
     "dlb_moe_topk_sum": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_void_p]),
 }
 

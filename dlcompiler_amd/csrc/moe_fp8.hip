@@ -15,6 +15,9 @@
 // counterpart there; its nearest precedent is the int8 per-token quantisation and
 // scale-in-epilogue GEMM of python/dlBLAS/dlblas/kernels/w8a8.py:102-106,275-335.
 //
+// The same kernel also runs unquantised bf16/f16 operands (QT = 1): the reference's own
+// fused_moe, with 16x16x32 MFMAs accumulating in place and no scales.
+//
 // GEMM mapping.  The MFMA runs "transposed": weight rows are the A operand (M index = output
 // column n), activations the B operand (N index = token row), so a lane's four accumulator
 // registers are four consecutive n of ONE token: the activation scale is a per-lane scalar
@@ -87,14 +90,14 @@ struct MoeGemmParams {
   const int32_t* sorted_ids;  // [num_mblocks * BM]
   const int32_t* expert_ids;  // [num_mblocks]
   int num_mblocks, num_ntiles, grid_real;
-  int K, N, KC;               // KC = K / 128
+  int K, N, KC;               // K = bytes per activation / weight row, KC = K / 128
   int topk, numel;            // flat slots = tokens * topk (also the pad sentinel)
   int num_tokens;
   int expert_offset;          // weights hold experts [expert_offset, expert_offset + E_local)
   int num_local;              // E_local
   int w_layout;               // 0: [E, N, K] row-major, 1: MFMA-operand order (see header)
   // gate_up flavour
-  unsigned char* hq;          // [num_mblocks * BM, I]
+  unsigned char* hq;          // [num_mblocks * BM, I] fp8, or 16-bit when QT = 1
   float* hs;                  // [num_mblocks * BM, I / 128]
   int I;
   // down flavour
@@ -109,11 +112,32 @@ __device__ __forceinline__ f32x4 mfma_fp8(const i32x8& a, const i32x8& b) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, z, 0, 0, 0, 0, 0, 0);
 }
 
+template <int DT>
+__device__ __forceinline__ f32x4 mfma_16bit(const i32x8& a, const i32x8& b, f32x4 c) {
+  // one 128-byte chunk = 64 elements = two 16x16x32 steps on the two operand halves
+  typedef __attribute__((ext_vector_type(4))) int i32x4;
+  const i32x4 a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
+  const i32x4 b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
+  if constexpr (DT == DLB_DTYPE_BF16) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a0),
+                                                __builtin_bit_cast(bf16x8, b0), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a1),
+                                                __builtin_bit_cast(bf16x8, b1), c, 0, 0, 0);
+  } else {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a0),
+                                               __builtin_bit_cast(f16x8, b0), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a1),
+                                               __builtin_bit_cast(f16x8, b1), c, 0, 0, 0);
+  }
+  return c;
+}
+
+// QT = 0: fp8 operands with block scales; QT = 1: 16-bit operands of type DT, no scales.
 // GATED = true : gate_up GEMM (N = 2I), tile = 128 gate cols + the matching 128 up cols,
 //                epilogue silu(gate) * up -> fp8 + per-128 scale, rows kept in sorted order.
 // GATED = false: down GEMM, tile = 256 cols, epilogue * routing weight -> out[slot, n].
 // BM = rows (routing slots) per workgroup = the alignment block of the routing (64 or 128).
-template <bool GATED, int DT, int BM>
+template <bool GATED, int DT, int BM, int QT>
 __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
   constexpr int kBM = BM;
   constexpr int MT = BM / 16;          // 16-token sub-tiles
@@ -166,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
       src_row = row0 + arow;
     }
     a_ptr = p.a + src_row * K;
-    as_ptr = p.a_scale + src_row * KC;
+    as_ptr = QT == 0 ? p.a_scale + src_row * KC : nullptr;
   }
 
   // ---- weight fragments: sub-tile j of this wave covers 16 output columns
@@ -205,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
       const int n = min(ncol[j] + c, p.N - 1);
       woff[j] = (uint32_t)n * (uint32_t)K + 16u * g;
     }
-    ws_ptr[j] = p.w_scale + ((int64_t)e * (p.N >> 7) + sblk[j]) * KC;
+    ws_ptr[j] = QT == 0 ? p.w_scale + ((int64_t)e * (p.N >> 7) + sblk[j]) * KC : nullptr;
   }
 
   f32x4 acc[MT][4];  // [token sub-tile mt][column sub-tile j]
@@ -232,13 +256,13 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
       const int kc = min(kc0 + (byte >> 7), KC - 1);
       areg[u] = *(const u32x4*)(a_ptr + kc * 128 + (byte & 127));
     }
-    if (aseg < SKC) asreg = as_ptr[min(kc0 + aseg, KC - 1)];
+    if (QT == 0 && aseg < SKC) asreg = as_ptr[min(kc0 + aseg, KC - 1)];
   };
   auto store_a = [&](int buf) {
     unsigned char* dst = a_lds[buf] + arow * kARow + aseg * (16 * AU);
 #pragma unroll
     for (int u = 0; u < AU; ++u) *(u32x4*)(dst + 16 * u) = areg[u];
-    if (aseg < SKC) as_lds[buf][aseg][arow] = asreg;
+    if (QT == 0 && aseg < SKC) as_lds[buf][aseg][arow] = asreg;
   };
   auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
     if (kc >= KC) return;
@@ -249,7 +273,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
       const u32x4 hi = *(const u32x4*)(src + w_hi_off + woff[j]);
       b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
                    (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-      bs[j] = ws_ptr[j][kc];
+      bs[j] = QT == 0 ? ws_ptr[j][kc] : 1.0f;
     }
   };
 
@@ -271,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     const u32x4 hi = *(const u32x4*)(src + 64);
     x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
               (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    as = as_lds[buf][ci][16 * mt + c];
+    as = QT == 0 ? as_lds[buf][ci][16 * mt + c] : 1.0f;
   };
   auto do_stage = [&](auto jtag, int st) {
     constexpr int J = decltype(jtag)::value;  // st % PD
@@ -299,16 +323,23 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
           } else if (ci + 1 < SKC) {
             if (ci + 1 < nchunks) read_x(buf, ci + 1, 0, xq[(t + 1) & 1], asq[(t + 1) & 1]);
           }
-          f32x4 pc[4];
+          if constexpr (QT == 0) {
+            f32x4 pc[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            pc[j] = mfma_fp8(breg[slot][j], xq[t & 1]);
-            acc[pm][j] += pp[j] * psc[j];
-          }
+            for (int j = 0; j < 4; ++j) {
+              pc[j] = mfma_fp8(breg[slot][j], xq[t & 1]);
+              acc[pm][j] += pp[j] * psc[j];
+            }
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            pp[j] = pc[j];
-            psc[j] = asq[t & 1] * bsreg[slot][j];
+            for (int j = 0; j < 4; ++j) {
+              pp[j] = pc[j];
+              psc[j] = asq[t & 1] * bsreg[slot][j];
+            }
+          } else {
+            (void)pm;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              acc[mt][j] = mfma_16bit<DT>(breg[slot][j], xq[t & 1], acc[mt][j]);
           }
         }
       }
@@ -334,7 +365,30 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
   for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[j];
 
   // ---- epilogues: lane holds token (16*mt + c), columns ncol[j] + 4*g + i
-  if (GATED) {
+  if (GATED && QT == 1) {
+    // rounding points of the reference pipeline (fused_moe.py:166,351-352): GEMM result,
+    // silu(gate) and the product are each rounded to the activation type
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int64_t orow = row0 + 16 * mt + c;
+      unsigned short* dst = (unsigned short*)p.hq + orow * p.I + nt * 128 + wave * 32 + 4 * g;
+#pragma unroll
+      for (int jg = 0; jg < 2; ++jg) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const unsigned int gu = Elem<DT>::pack(acc[mt][jg][i], acc[mt][jg + 2][i]);
+          const float gate = Elem<DT>::lo(gu), up = Elem<DT>::hi(gu);
+          const float sg = Elem<DT>::lo(Elem<DT>::pack(gate / (1.0f + __expf(-gate)), 0.0f));
+          v[i] = sg * up;
+        }
+        u32x2 o2;
+        o2[0] = Elem<DT>::pack(v[0], v[1]);
+        o2[1] = Elem<DT>::pack(v[2], v[3]);
+        *(u32x2*)(dst + 16 * jg) = o2;
+      }
+    }
+  } else if (GATED) {
     float h[MT][2][4];
     float amax[MT];
 #pragma unroll
@@ -421,18 +475,6 @@ __global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restri
   out[i] = r;
 }
 
-int check_gemm_common(const void* a, const void* a_scale, const void* w, const void* w_scale,
-                      const void* sorted_ids, const void* expert_ids, int num_mblocks, int K,
-                      int N) {
-  if (num_mblocks < 0 || K < 1 || N < 1) return DLB_ERR_BAD_ARG;
-  if (num_mblocks == 0) return DLB_OK;
-  if (!a || !a_scale || !w || !w_scale || !sorted_ids || !expert_ids) return DLB_ERR_BAD_ARG;
-  if (K % 128 != 0 || N % 128 != 0) return DLB_ERR_UNSUPPORTED;
-  if ((int64_t)N * K >= (int64_t)0xffffffffu) return DLB_ERR_UNSUPPORTED;  // 32-bit lane offsets
-  if (!aligned16(a) || !aligned16(w)) return DLB_ERR_UNSUPPORTED;
-  return DLB_OK;
-}
-
 }  // namespace
 }  // namespace dlb
 
@@ -463,6 +505,72 @@ extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs,
   return launch_status();
 }
 
+namespace dlb {
+namespace {
+
+template <bool GATED, int QT>
+int launch_moe_gemm(const MoeGemmParams& p, int dtype, int block_m, hipStream_t s) {
+  const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
+#define DLB_LAUNCH_GEMM(DT_, BM_) \
+  hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, BM_, QT>), dim3(grid), dim3(256), 0, s, p)
+  if (dtype == DLB_DTYPE_BF16) {
+    if (block_m == 128) DLB_LAUNCH_GEMM(DLB_DTYPE_BF16, 128);
+    else DLB_LAUNCH_GEMM(DLB_DTYPE_BF16, 64);
+  } else if (dtype == DLB_DTYPE_F16) {
+    if (block_m == 128) DLB_LAUNCH_GEMM(DLB_DTYPE_F16, 128);
+    else DLB_LAUNCH_GEMM(DLB_DTYPE_F16, 64);
+  } else {
+    return DLB_ERR_UNSUPPORTED;
+  }
+#undef DLB_LAUNCH_GEMM
+  return launch_status();
+}
+
+// shared argument checks and parameter block of the four grouped-GEMM entry points;
+// elem = bytes per operand element (1 for fp8, 2 for bf16/f16)
+int fill_gemm_params(MoeGemmParams& p, bool gated, int elem, const void* a, const float* a_scale,
+                     const void* w, const float* w_scale, const int32_t* sorted_ids,
+                     const int32_t* expert_ids, int num_mblocks, int block_m, int num_tokens,
+                     int topk, int H, int I, int expert_offset, int num_local_experts,
+                     int w_layout) {
+  const int Kel = gated ? H : I;       // reduction length (elements)
+  const int N = gated ? 2 * I : H;     // weight rows per expert
+  if (num_mblocks < 0 || H < 1 || I < 1) return DLB_ERR_BAD_ARG;
+  if (num_mblocks == 0) return DLB_OK;
+  if (!a || !w || !sorted_ids || !expert_ids) return DLB_ERR_BAD_ARG;
+  if (elem == 1 && (!a_scale || !w_scale)) return DLB_ERR_BAD_ARG;
+  if (num_tokens < 1 || topk < 1 || num_local_experts < 1) return DLB_ERR_BAD_ARG;
+  if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
+  // a row must be a whole number of 128-byte chunks; output tiles are 128 columns wide
+  if ((Kel * elem) % 128 != 0 || I % 128 != 0 || H % 128 != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(a) || !aligned16(w)) return DLB_ERR_UNSUPPORTED;
+  if ((int64_t)N * Kel * elem >= (int64_t)0xffffffffu) return DLB_ERR_UNSUPPORTED;  // 32-bit lane offsets
+  p = MoeGemmParams{};
+  p.a = (const unsigned char*)a;
+  p.a_scale = a_scale;
+  p.w = (const unsigned char*)w;
+  p.w_scale = w_scale;
+  p.sorted_ids = sorted_ids;
+  p.expert_ids = expert_ids;
+  p.num_mblocks = num_mblocks;
+  p.num_ntiles = gated ? I / 128 : (int)ceil_div(H, 256);
+  p.K = Kel * elem;
+  p.N = N;
+  p.KC = p.K / 128;
+  p.topk = topk;
+  p.numel = num_tokens * topk;
+  p.num_tokens = num_tokens;
+  p.expert_offset = expert_offset;
+  p.num_local = num_local_experts;
+  p.w_layout = w_layout ? 1 : 0;
+  p.I = I;
+  p.grid_real = p.num_mblocks * p.num_ntiles;
+  return DLB_OK;
+}
+
+}  // namespace
+}  // namespace dlb
+
 extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q,
                                         const float* w1s, const int32_t* sorted_ids,
                                         const int32_t* expert_ids, int num_mblocks, int block_m,
@@ -470,41 +578,16 @@ extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const v
                                         int expert_offset, int num_local_experts, int w_layout,
                                         void* hq, float* hs, void* stream) {
   using namespace dlb;
-  const int st = check_gemm_common(xq, xs, w1q, w1s, sorted_ids, expert_ids, num_mblocks, H, I);
+  MoeGemmParams p;
+  const int st = fill_gemm_params(p, true, 1, xq, xs, w1q, w1s, sorted_ids, expert_ids,
+                                  num_mblocks, block_m, num_tokens, topk, H, I, expert_offset,
+                                  num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
-  if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
-  if (num_tokens < 1 || topk < 1 || num_local_experts < 1 || !hq || !hs) return DLB_ERR_BAD_ARG;
+  if (!hq || !hs) return DLB_ERR_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(hq) & 3u) != 0) return DLB_ERR_UNSUPPORTED;
-  MoeGemmParams p = {};
-  p.a = (const unsigned char*)xq;
-  p.a_scale = xs;
-  p.w = (const unsigned char*)w1q;
-  p.w_scale = w1s;
-  p.sorted_ids = sorted_ids;
-  p.expert_ids = expert_ids;
-  p.num_mblocks = num_mblocks;
-  p.num_ntiles = I / 128;
-  p.K = H;
-  p.N = 2 * I;
-  p.KC = H / 128;
-  p.topk = topk;
-  p.numel = num_tokens * topk;
-  p.num_tokens = num_tokens;
-  p.expert_offset = expert_offset;
-  p.num_local = num_local_experts;
-  p.w_layout = w_layout ? 1 : 0;
   p.hq = (unsigned char*)hq;
   p.hs = hs;
-  p.I = I;
-  p.grid_real = p.num_mblocks * p.num_ntiles;
-  const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
-  if (block_m == 128)
-    hipLaunchKernelGGL((moe_gemm_fp8_kernel<true, DLB_DTYPE_BF16, 128>), dim3(grid), dim3(256), 0,
-                       (hipStream_t)stream, p);
-  else
-    hipLaunchKernelGGL((moe_gemm_fp8_kernel<true, DLB_DTYPE_BF16, 64>), dim3(grid), dim3(256), 0,
-                       (hipStream_t)stream, p);
-  return launch_status();
+  return launch_moe_gemm<true, 0>(p, DLB_DTYPE_BF16, block_m, (hipStream_t)stream);
 }
 
 extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q,
@@ -512,52 +595,54 @@ extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void
                                      const int32_t* expert_ids, const float* topk_weights,
                                      int num_mblocks, int block_m, int num_tokens, int topk,
                                      int H, int I, int expert_offset, int num_local_experts,
-                                     int w_layout, void* out,
-                                     int out_dtype, void* stream) {
+                                     int w_layout, void* out, int out_dtype, void* stream) {
   using namespace dlb;
-  const int st = check_gemm_common(hq, hs, w2q, w2s, sorted_ids, expert_ids, num_mblocks, I, H);
+  MoeGemmParams p;
+  const int st = fill_gemm_params(p, false, 1, hq, hs, w2q, w2s, sorted_ids, expert_ids,
+                                  num_mblocks, block_m, num_tokens, topk, H, I, expert_offset,
+                                  num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
-  if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
-  if (num_tokens < 1 || topk < 1 || num_local_experts < 1 || !out || !topk_weights)
-    return DLB_ERR_BAD_ARG;
+  if (!out || !topk_weights) return DLB_ERR_BAD_ARG;
   if ((reinterpret_cast<uintptr_t>(out) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
-  MoeGemmParams p = {};
-  p.a = (const unsigned char*)hq;
-  p.a_scale = hs;
-  p.w = (const unsigned char*)w2q;
-  p.w_scale = w2s;
-  p.sorted_ids = sorted_ids;
-  p.expert_ids = expert_ids;
-  p.num_mblocks = num_mblocks;
-  p.num_ntiles = (int)ceil_div(H, 256);
-  p.K = I;
-  p.N = H;
-  p.KC = I / 128;
-  p.topk = topk;
-  p.numel = num_tokens * topk;
-  p.num_tokens = num_tokens;
-  p.expert_offset = expert_offset;
-  p.num_local = num_local_experts;
-  p.w_layout = w_layout ? 1 : 0;
   p.out = out;
   p.topk_w = topk_weights;
-  p.I = I;
-  p.grid_real = p.num_mblocks * p.num_ntiles;
-  const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
-#define DLB_LAUNCH_DOWN(DT_, BM_)                                                              \
-  hipLaunchKernelGGL((moe_gemm_fp8_kernel<false, DT_, BM_>), dim3(grid), dim3(256), 0,         \
-                     (hipStream_t)stream, p)
-  if (out_dtype == DLB_DTYPE_BF16) {
-    if (block_m == 128) DLB_LAUNCH_DOWN(DLB_DTYPE_BF16, 128);
-    else DLB_LAUNCH_DOWN(DLB_DTYPE_BF16, 64);
-  } else if (out_dtype == DLB_DTYPE_F16) {
-    if (block_m == 128) DLB_LAUNCH_DOWN(DLB_DTYPE_F16, 128);
-    else DLB_LAUNCH_DOWN(DLB_DTYPE_F16, 64);
-  } else {
-    return DLB_ERR_UNSUPPORTED;
-  }
-#undef DLB_LAUNCH_DOWN
-  return launch_status();
+  return launch_moe_gemm<false, 0>(p, out_dtype, block_m, (hipStream_t)stream);
+}
+
+extern "C" int dlb_moe_gemm_16bit_gate_up(const void* x, const void* w1,
+                                          const int32_t* sorted_ids, const int32_t* expert_ids,
+                                          int num_mblocks, int block_m, int num_tokens, int topk,
+                                          int H, int I, int expert_offset, int num_local_experts,
+                                          int w_layout, void* act, int dtype, void* stream) {
+  using namespace dlb;
+  MoeGemmParams p;
+  const int st = fill_gemm_params(p, true, 2, x, nullptr, w1, nullptr, sorted_ids, expert_ids,
+                                  num_mblocks, block_m, num_tokens, topk, H, I, expert_offset,
+                                  num_local_experts, w_layout);
+  if (st != DLB_OK || num_mblocks == 0) return st;
+  if (!act) return DLB_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(act) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  p.hq = (unsigned char*)act;
+  return launch_moe_gemm<true, 1>(p, dtype, block_m, (hipStream_t)stream);
+}
+
+extern "C" int dlb_moe_gemm_16bit_down(const void* act, const void* w2,
+                                       const int32_t* sorted_ids, const int32_t* expert_ids,
+                                       const float* topk_weights, int num_mblocks, int block_m,
+                                       int num_tokens, int topk, int H, int I, int expert_offset,
+                                       int num_local_experts, int w_layout, void* out, int dtype,
+                                       void* stream) {
+  using namespace dlb;
+  MoeGemmParams p;
+  const int st = fill_gemm_params(p, false, 2, act, nullptr, w2, nullptr, sorted_ids, expert_ids,
+                                  num_mblocks, block_m, num_tokens, topk, H, I, expert_offset,
+                                  num_local_experts, w_layout);
+  if (st != DLB_OK || num_mblocks == 0) return st;
+  if (!out || !topk_weights) return DLB_ERR_BAD_ARG;
+  if ((reinterpret_cast<uintptr_t>(out) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  p.out = out;
+  p.topk_w = topk_weights;
+  return launch_moe_gemm<false, 1>(p, dtype, block_m, (hipStream_t)stream);
 }
 
 extern "C" int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk,

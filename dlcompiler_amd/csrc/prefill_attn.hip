@@ -16,6 +16,8 @@
 //   * the exponent runs in base 2 with the softmax scale folded into one FMA;
 //   * fully masked tiles are skipped per wave and only diagonal tiles pay for the mask; the
 //     heaviest query tiles are launched first.
+#include <type_traits>
+
 #include "common.h"
 
 namespace dlb {
@@ -69,18 +71,20 @@ constexpr int kThreads = 256;
 
 template <int D>
 struct Smem {
-  static constexpr int kRowBytes = D * 2 + 16;      // K: [64][D] + pad
+  static constexpr int kRowBytes = D * 2;           // K: [64][D], 16-byte chunks XOR-swizzled
   static constexpr int kBytes = kTileN * kRowBytes;
   static constexpr int vRowBytes = kTileN * 2 + 16;  // V^T: [D][64] + pad
   static constexpr int vBytes = D * vRowBytes;
   static constexpr int stage = kBytes + vBytes;
 };
 
+#ifndef DLB_PF_OCC
+#define DLB_PF_OCC 2
+#endif
 template <int DT, int D>
-__global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int KS = D / 16;  // MFMA k-steps over the head dim for S^T
   constexpr int MT = D / 32;  // 32-row tiles of O^T
-  constexpr int KLD = (kTileN * D / 8) / kThreads;  // 16-byte K loads per thread per tile
   constexpr int VUNITS = (kTileN / 4) * (D / 8);    // (4 keys x 8 dims) units per tile
   constexpr int VLD = (VUNITS + kThreads - 1) / kThreads;
   constexpr int DG = D / 8;
@@ -120,62 +124,70 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
 
   const int kv_end = min(L, q0 + kBlockM);            // keys this workgroup needs
   const int ntiles = (kv_end + kTileN - 1) / kTileN;
+  // tiles below this index lie entirely under the diagonal for every wave of the workgroup
+  // (q0 is a multiple of 128): no mask, no clamping of key rows
+  const int nfull = q0 / kTileN;
   const int wave_last_row = q0 + 32 * wave + 31;
-  const int wave_first_row = q0 + 32 * wave;
 
-  // ---- global -> register staging of one K/V tile
-  u32x4 kreg[KLD];
-  u32x4 vreg[VLD][4];
-  auto load_tile = [&](int t0) {
+  // ---- global -> register staging of one K/V tile.  Per-thread base pointers are formed
+  // once; a tile adds a workgroup-uniform offset.  CLAMP (tiles that may run past the
+  // sequence) redirects rows >= L to row L-1 so nothing outside the sequence is read.
+  // K goes global -> LDS directly (global_load_lds_dwordx4: lane l's 16 bytes land at
+  // base + 16*l, so one wave instruction fills 1 KB = 1024 / (2*D) rows).  Rows are stored
+  // unpadded; bank conflicts are avoided by letting lane (row r, position c) fetch global
+  // chunk c ^ (r & 15): a reader that wants chunk c of row r reads position c ^ (r & 15).
+  constexpr int KRPI = 1024 / (2 * D);            // rows per wave instruction
+  constexpr int KINS = kTileN / KRPI / 4;         // instructions per wave and tile
+  const int k_lrow = lane / DG;                   // row inside an instruction
+  const int k_pos = lane % DG;                    // 16-byte position inside the row
+  const unsigned char* kbytes = (const unsigned char*)kb;
+  const unsigned char* vbase = (const unsigned char*)vb + ((tok0 + 4 * (tid / DG)) * p.v_st + 8 * (tid % DG)) * 2;
+  const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
+  const bool v_active = (VUNITS >= kThreads) || (tid < VUNITS);
+  u32x4 vreg[4];
+  static_assert(VLD == 1, "one (4 keys x 8 dims) V unit per thread");
+  auto load_tile = [&](auto clamp_tag, int t0, int buf) {
+    constexpr bool CLAMP = decltype(clamp_tag)::value;
+    unsigned char* ks = smem + buf * SM::stage;
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) {
-      const int u = i * kThreads + tid;
-      const int row = u / DG, cg = u % DG;
-      const int key = min(t0 + row, L - 1);
-      kreg[i] = *(const u32x4*)(kb + (tok0 + key) * p.k_st + 8 * cg);
+    for (int i = 0; i < KINS; ++i) {
+      const int q = 4 * i + wave;                 // which 1 KB slice of the tile
+      const int r = q * KRPI + k_lrow;            // key row inside the tile
+      int key = t0 + r;
+      if (CLAMP) key = min(key, L - 1);
+      const unsigned char* src = kbytes + (tok0 + key) * k_row_bytes + ((k_pos ^ (r & (DG - 1))) << 4);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(ks + q * 1024),
+                                       16, 0, 0);
     }
+    if (v_active) {
 #pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const int u = i * kThreads + tid;
-      if (VUNITS % kThreads == 0 || u < VUNITS) {
-        const int dg = u % DG, kg = u / DG;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int key = min(t0 + 4 * kg + r, L - 1);
-          vreg[i][r] = *(const u32x4*)(vb + (tok0 + key) * p.v_st + 8 * dg);
-        }
+      for (int r = 0; r < 4; ++r) {
+        int row = t0 + r;  // + 4 * (tid / DG) is in vbase
+        if (CLAMP) row = min(row + 4 * (tid / DG), L - 1) - 4 * (tid / DG);
+        vreg[r] = *(const u32x4*)(vbase + row * v_row_bytes);
       }
     }
   };
+  // LDS addresses of this thread's staging slots (tile-independent)
+  const int st_kg = tid / DG, st_dg = tid % DG;
+  // key = 32*nt + 16*st + 8*a + 4*h + r  ->  position 32*nt + 16*st + 8*h + 4*a + r
+  const int st_unit = ((st_kg >> 2) << 1) | (st_kg & 1);  // 16-byte unit 4*nt + 2*st + h
+  const int st_half = (st_kg >> 1) & 1;                   // 8-byte half a
   auto store_tile = [&](int buf) {
-    unsigned char* ks = smem + buf * SM::stage;
-    unsigned char* vs = ks + SM::kBytes;
+    unsigned char* vs = smem + buf * SM::stage + SM::kBytes;
+    if (v_active) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) {
-      const int u = i * kThreads + tid;
-      const int row = u / DG, cg = u % DG;
-      *(u32x4*)(ks + row * SM::kRowBytes + cg * 16) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VLD; ++i) {
-      const int u = i * kThreads + tid;
-      if (VUNITS % kThreads == 0 || u < VUNITS) {
-        const int dg = u % DG, kg = u / DG;
-        // key = 32*nt + 16*st + 8*a + 4*h + r  ->  position 32*nt + 16*st + 8*h + 4*a + r
-        const int unit = ((kg >> 2) << 1) | (kg & 1);  // 4*nt + 2*st + h
-        const int half = (kg >> 1) & 1;                // a
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const unsigned int lo01 = __builtin_amdgcn_perm(vreg[i][1][w], vreg[i][0][w], 0x05040100u);
-          const unsigned int lo23 = __builtin_amdgcn_perm(vreg[i][3][w], vreg[i][2][w], 0x05040100u);
-          const unsigned int hi01 = __builtin_amdgcn_perm(vreg[i][1][w], vreg[i][0][w], 0x07060302u);
-          const unsigned int hi23 = __builtin_amdgcn_perm(vreg[i][3][w], vreg[i][2][w], 0x07060302u);
-          const int d0 = 8 * dg + 2 * w;
-          const int sw = ((d0 >> 4) & 3) << 1;
-          unsigned char* row = vs + d0 * SM::vRowBytes + ((unit ^ sw) << 4) + (half << 3);
-          *(u32x2*)(row) = u32x2{lo01, lo23};
-          *(u32x2*)(row + SM::vRowBytes) = u32x2{hi01, hi23};
-        }
+      for (int w = 0; w < 4; ++w) {
+        const unsigned int lo01 = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], 0x05040100u);
+        const unsigned int lo23 = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], 0x05040100u);
+        const unsigned int hi01 = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], 0x07060302u);
+        const unsigned int hi23 = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], 0x07060302u);
+        const int d0 = 8 * st_dg + 2 * w;
+        const int sw = (d0 >> 4) & 7;  // same for d0 and d0 + 1; spreads the 16 dim groups
+        unsigned char* row = vs + d0 * SM::vRowBytes + ((st_unit ^ sw) << 4) + (st_half << 3);
+        *(u32x2*)(row) = u32x2{lo01, lo23};
+        *(u32x2*)(row + SM::vRowBytes) = u32x2{hi01, hi23};
       }
     }
   };
@@ -185,95 +197,124 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[mt][i] = 0.0f;
+  // m_run is the exponent reference in the log2 domain.  It follows the running maximum
+  // lazily: the accumulators are rescaled only when a row maximum exceeds it by more than
+  // kRescaleGap, so between rescales probabilities stay below 2^kRescaleGap -- exact in the
+  // end (the same factor cancels in O / l), and it removes the per-tile rescale of O.
+  constexpr float kRescaleGap = 8.0f;
   float m_run = -__builtin_inff();
   float l_run = 0.0f;  // this lane half's share of the denominator
+  const float cs = p.scale_log2e;
 
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-
-  for (int j = 0; j < ntiles; ++j) {
+  // one K/V tile against this wave's 32 queries; MASK: apply the causal mask
+  auto process_tile = [&](auto mask_tag, int j) {
+    constexpr bool MASK = decltype(mask_tag)::value;
     const int t0 = j * kTileN;
-    const bool more = (j + 1 < ntiles);
-    if (more) load_tile(t0 + kTileN);
+    if (MASK && t0 > wave_last_row) return;  // wave-uniform: tile entirely above the diagonal
+    const unsigned char* ks = smem + (j & 1) * SM::stage;
+    const unsigned char* vs = ks + SM::kBytes;
 
-    if (t0 <= wave_last_row) {  // wave-uniform: tile not entirely above the diagonal
-      const unsigned char* ks = smem + (j & 1) * SM::stage;
-      const unsigned char* vs = ks + SM::kBytes;
-
-      // ---- S^T = K . Q^T : two 32-key tiles x 32 queries
-      f32x16 s[2];
+    // ---- S^T = K . Q^T : two 32-key tiles x 32 queries (raw scores)
+    f32x16 s[2];
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
-        const unsigned char* krow = ks + (32 * nt + col) * SM::kRowBytes + 16 * hh;
+      for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
+      const int krow_i = 32 * nt + col;
+      const unsigned char* krow = ks + krow_i * SM::kRowBytes;
+      const int ksw = krow_i & (DG - 1);
 #pragma unroll
-        for (int kstep = 0; kstep < KS; ++kstep) {
-          const u32x4 a = *(const u32x4*)(krow + 32 * kstep);
-          s[nt] = Mma32<DT>::run(a, qf[kstep], s[nt]);
-        }
+      for (int kstep = 0; kstep < KS; ++kstep) {
+        const u32x4 a = *(const u32x4*)(krow + (((2 * kstep + hh) ^ ksw) << 4));
+        s[nt] = Mma32<DT>::run(a, qf[kstep], s[nt]);
       }
+    }
 
-      // ---- causal mask (diagonal tiles only) and running max, log2 domain
-      const bool diag = (t0 + kTileN - 1 > wave_first_row);
-      float mloc = -__builtin_inff();
+    // ---- causal mask and tile maximum of the raw scores (scale > 0 commutes with max)
+    float mloc = -__builtin_inff();
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float x = s[nt][i] * p.scale_log2e;
-          if (diag) {
-            const int key = t0 + 32 * nt + 8 * (i >> 2) + 4 * hh + (i & 3);
-            x = (key <= qrow) ? x : -__builtin_inff();
-          }
-          s[nt][i] = x;
-          mloc = fmaxf(mloc, x);
+      for (int i = 0; i < 16; ++i) {
+        if (MASK) {
+          const int key = t0 + 32 * nt + 8 * (i >> 2) + 4 * hh + (i & 3);
+          s[nt][i] = (key <= qrow) ? s[nt][i] : -__builtin_inff();
         }
+        mloc = fmaxf(mloc, s[nt][i]);
       }
-      mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-      const float m_new = fmaxf(m_run, mloc);  // finite from tile 0 on (key 0 is always visible)
+    }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * cs;
+    if (__any(mloc > m_run + kRescaleGap)) {
+      const float m_new = fmaxf(m_run, mloc);  // finite from tile 0 on (key 0 is visible)
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       m_run = m_new;
-      float psum = 0.0f;
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float e = __builtin_amdgcn_exp2f(s[nt][i] - m_new);
-          s[nt][i] = e;
-          psum += e;
-        }
-      }
-      l_run = l_run * alpha + psum;
+      l_run *= alpha;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
+    }
+    float psum = 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][i], cs, -m_run));
+        s[nt][i] = e;
+        psum += e;
+      }
+    }
+    l_run += psum;
 
-      // ---- O^T += V^T . P^T ; step (nt, st) consumes registers 8*st .. 8*st+7 of s[nt]
+    // ---- O^T += V^T . P^T ; step (nt, st) consumes registers 8*st .. 8*st+7 of s[nt]
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          u32x4 pf;
-          pf[0] = Mma32<DT>::pack2(s[nt][8 * st + 0], s[nt][8 * st + 1]);
-          pf[1] = Mma32<DT>::pack2(s[nt][8 * st + 2], s[nt][8 * st + 3]);
-          pf[2] = Mma32<DT>::pack2(s[nt][8 * st + 4], s[nt][8 * st + 5]);
-          pf[3] = Mma32<DT>::pack2(s[nt][8 * st + 6], s[nt][8 * st + 7]);
-          const int unit = 4 * nt + 2 * st + hh;
+      for (int st = 0; st < 2; ++st) {
+        u32x4 pf;
+        pf[0] = Mma32<DT>::pack2(s[nt][8 * st + 0], s[nt][8 * st + 1]);
+        pf[1] = Mma32<DT>::pack2(s[nt][8 * st + 2], s[nt][8 * st + 3]);
+        pf[2] = Mma32<DT>::pack2(s[nt][8 * st + 4], s[nt][8 * st + 5]);
+        pf[3] = Mma32<DT>::pack2(s[nt][8 * st + 6], s[nt][8 * st + 7]);
+        const int unit = 4 * nt + 2 * st + hh;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            const int d = 32 * mt + col;
-            const int sw = ((d >> 4) & 3) << 1;
-            const u32x4 a = *(const u32x4*)(vs + d * SM::vRowBytes + ((unit ^ sw) << 4));
-            o[mt] = Mma32<DT>::run(a, pf, o[mt]);
-          }
+        for (int mt = 0; mt < MT; ++mt) {
+          const int d = 32 * mt + col;
+          const int sw = (d >> 4) & 7;
+          const u32x4 a = *(const u32x4*)(vs + d * SM::vRowBytes + ((unit ^ sw) << 4));
+          o[mt] = Mma32<DT>::run(a, pf, o[mt]);
         }
       }
     }
+  };
 
+  using NoClamp = std::integral_constant<bool, false>;
+  using Clamp = std::integral_constant<bool, true>;
+  // vmcnt(0): the direct-to-LDS loads of this wave have landed before the barrier publishes
+  // the buffer (encoding: vmcnt = 0, expcnt / lgkmcnt left at their maxima)
+  auto wait_dma = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
+  if (nfull > 0) load_tile(NoClamp{}, 0, 0); else load_tile(Clamp{}, 0, 0);
+  store_tile(0);
+  wait_dma();
+  __syncthreads();
+
+  int j = 0;
+  // tiles under the diagonal whose successor is also under it: nothing to mask or clamp
+  for (; j + 1 < nfull; ++j) {
+    load_tile(NoClamp{}, (j + 1) * kTileN, (j + 1) & 1);
+    process_tile(std::integral_constant<bool, false>{}, j);
+    store_tile((j + 1) & 1);
+    wait_dma();
+    __syncthreads();
+  }
+  // last unmasked tile (its successor may run past the sequence), then the diagonal tiles
+  for (; j < ntiles; ++j) {
+    const bool more = (j + 1 < ntiles);
+    if (more) load_tile(Clamp{}, (j + 1) * kTileN, (j + 1) & 1);
+    if (j < nfull) process_tile(std::integral_constant<bool, false>{}, j);
+    else process_tile(std::integral_constant<bool, true>{}, j);
     if (more) store_tile((j + 1) & 1);
+    wait_dma();
     __syncthreads();
   }
 

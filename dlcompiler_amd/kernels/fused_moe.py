@@ -42,16 +42,21 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
     return xq, xs
 
 
-def shuffle_moe_weight_fp8(w_q: torch.Tensor) -> torch.Tensor:
-    """Re-arrange fp8 expert weights ``[E, N, K]`` into MFMA-operand order (done once, when the
-    weights are loaded): per expert, 16-row tile and 128-byte K chunk one 2 KB block laid out
-    ``[half][lane][16 bytes]`` with ``lane = 16 * (k_piece) + row``, so every operand fetch of
-    the grouped GEMM is a contiguous 1 KB access.  Same bytes and the same block scales."""
-    E, N, K = w_q.shape
-    assert w_q.dtype == torch.float8_e4m3fn and N % 16 == 0 and K % 128 == 0
-    b = w_q.contiguous().view(torch.uint8).view(E, N // 16, 16, K // 128, 2, 4, 16)
+def shuffle_moe_weight(w: torch.Tensor) -> torch.Tensor:
+    """Re-arrange expert weights ``[E, N, K]`` (fp8, bf16 or f16) into MFMA-operand order (done
+    once, when the weights are loaded): per expert, 16-row tile and 128-byte K chunk one 2 KB
+    block laid out ``[half][lane][16 bytes]`` with ``lane = 16 * (k_piece) + row``, so every
+    operand fetch of the grouped GEMM is a contiguous 1 KB access.  Same bytes (and for fp8
+    the same block scales); shape and dtype are kept."""
+    E, N, K = w.shape
+    kb = K * w.element_size()
+    assert N % 16 == 0 and kb % 128 == 0
+    b = w.contiguous().view(torch.uint8).view(E, N // 16, 16, kb // 128, 2, 4, 16)
     # (e, nb, row c, kc, half h, piece g, byte) -> (e, nb, kc, h, g, c, byte)
-    return b.permute(0, 1, 3, 4, 5, 2, 6).contiguous().view(E, N, K).view(torch.float8_e4m3fn)
+    return b.permute(0, 1, 3, 4, 5, 2, 6).contiguous().view(E, N, kb).view(w.dtype).view(E, N, K)
+
+
+shuffle_moe_weight_fp8 = shuffle_moe_weight
 
 
 def get_start_end(topk_idx: torch.Tensor, sorted_idx: torch.Tensor, num_experts: int):
@@ -149,4 +154,66 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
                                   _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_topk_sum")
         hook(None)
+    return out
+
+
+def fused_moe(hidden_states: torch.Tensor,
+              w1: torch.Tensor,
+              w2: torch.Tensor,
+              topk_weights: torch.Tensor,
+              topk_ids: torch.Tensor,
+              topk: int,
+              expert_offset: int = 0,
+              num_experts: int = None,
+              renormalize: bool = False,
+              weights_shuffled: bool = False) -> torch.Tensor:
+    """fused moe -- signature and semantics of ``dlblas.kernels.fused_moe.fused_moe``
+    (reference: fused_moe.py:296-376): ``w1`` [E, 2I, H] (gate rows first), ``w2`` [E, H, I],
+    bf16/f16; routing slots are grouped by expert, the gate_up grouped GEMM runs with the
+    SiLU-and-mul fused into its epilogue (same rounding points as the reference), the down
+    grouped GEMM applies the routing weight and the top-k slots are summed.
+    ``weights_shuffled`` is this package's extension (see :func:`shuffle_moe_weight`)."""
+    _lib.require_cuda(hidden_states, w1, w2, topk_weights, topk_ids)
+    M = hidden_states.size(0)
+    E, N, _ = w1.shape
+    H = hidden_states.size(1)
+    I = N // 2
+    assert w1.shape == (E, 2 * I, H) and w2.shape == (E, H, I)
+    assert hidden_states.dtype == w1.dtype == w2.dtype
+    assert w1.is_contiguous() and w2.is_contiguous()
+    if num_experts is None:
+        num_experts = E
+    dev, dt = hidden_states.device, hidden_states.dtype
+    if M == 0:
+        return hidden_states.new_empty((0, H))
+    if hidden_states.stride(1) != 1 or hidden_states.stride(0) != H:
+        hidden_states = hidden_states.contiguous()
+
+    if renormalize:
+        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+    topk_weights = topk_weights.to(torch.float32).contiguous()
+
+    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, _ALIGN_BLOCK, num_experts)
+    num_mblocks = expert_ids.numel()
+    act = torch.empty((num_mblocks * _ALIGN_BLOCK, I), dtype=dt, device=dev)
+    full = (expert_offset == 0 and num_experts == E)
+    slots = (torch.empty if full else torch.zeros)((M * topk, H), dtype=dt, device=dev)
+    out = torch.empty((M, H), dtype=dt, device=dev)
+    lib = _lib.load()
+    code = _lib.torch_dtype_code(dt)
+    stream = _lib.current_stream_ptr(dev)
+    with torch.cuda.device(dev):
+        st = lib.dlb_moe_gemm_16bit_gate_up(hidden_states.data_ptr(), w1.data_ptr(),
+                                            sorted_ids.data_ptr(), expert_ids.data_ptr(),
+                                            num_mblocks, _ALIGN_BLOCK, M, topk, H, I,
+                                            expert_offset, E, int(weights_shuffled),
+                                            act.data_ptr(), code, stream)
+        _lib.check(st, "dlb_moe_gemm_16bit_gate_up")
+        st = lib.dlb_moe_gemm_16bit_down(act.data_ptr(), w2.data_ptr(), sorted_ids.data_ptr(),
+                                         expert_ids.data_ptr(), topk_weights.data_ptr(),
+                                         num_mblocks, _ALIGN_BLOCK, M, topk, H, I, expert_offset,
+                                         E, int(weights_shuffled), slots.data_ptr(), code, stream)
+        _lib.check(st, "dlb_moe_gemm_16bit_down")
+        st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), M, topk, H, code, stream)
+        _lib.check(st, "dlb_moe_topk_sum")
     return out

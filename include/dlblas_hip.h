@@ -191,6 +191,29 @@ int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q, cons
 int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk, int64_t N,
                      int dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Unquantised (bf16/f16) fused MoE: the reference's own fused_moe pipeline,
+ * kernels/fused_moe.py:82-235 (grouped GEMM kernel + launcher) and :334-373 (the two calls).
+ * Same routing inputs, tile height and weight layouts as the fp8 GEMMs above (w_layout 1 is
+ * the same byte re-arrangement applied to the 2-byte elements: 128-byte chunks = 64 elements).
+ *   gate_up: act[r, :] = round(silu(round(x_t W_gate^T)) * round(x_t W_up^T)) for the slot at
+ *            sorted position r -- the rounding points of the reference (GEMM result stored in
+ *            the activation dtype, then F.silu(...) * up, :351-352); act [num_mblocks*block_m, I]
+ *   down:    out[slot, :] = round((act_r W_down^T) * topk_weights[slot]), out [T * topk, H]
+ * x [T, H], w1 [E_local, 2I, H], w2 [E_local, H, I], all of `dtype`; H % 128 == 0, I % 128 == 0.
+ * Follow with dlb_moe_topk_sum.
+ * ---------------------------------------------------------------------------------------- */
+int dlb_moe_gemm_16bit_gate_up(const void* x, const void* w1, const int32_t* sorted_ids,
+                               const int32_t* expert_ids, int num_mblocks, int block_m,
+                               int num_tokens, int topk, int H, int I, int expert_offset,
+                               int num_local_experts, int w_layout, void* act, int dtype,
+                               void* stream);
+int dlb_moe_gemm_16bit_down(const void* act, const void* w2, const int32_t* sorted_ids,
+                            const int32_t* expert_ids, const float* topk_weights,
+                            int num_mblocks, int block_m, int num_tokens, int topk, int H, int I,
+                            int expert_offset, int num_local_experts, int w_layout, void* out,
+                            int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

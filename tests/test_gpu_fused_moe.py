@@ -1,0 +1,85 @@
+"""GPU parity: fused_moe (bf16/f16, the reference's own operator) and get_start_end vs the CPU
+oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import fused_moe as ofm
+from oracle import moe_gating as og
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(T, H, I, E, k, seed, dtype, uniform=False):
+    g = torch.Generator().manual_seed(seed)
+    if uniform:      # the reference fixtures: (rand - 0.5) / 2, test_fused_moe.py:190-205
+        mk = lambda *shape: ((torch.rand(shape, generator=g) - 0.5) / 2).to(dtype)
+        logits = torch.rand((T, E), generator=g)
+    else:
+        mk = lambda *shape: (torch.randn(shape, generator=g) * 0.03).to(dtype)
+        logits = torch.randn((T, E), generator=g)
+    x = mk(T, H) if uniform else torch.randn((T, H), generator=g).to(dtype)
+    w1, w2 = mk(E, 2 * I, H), mk(E, H, I)
+    tw, ids = og.topk_softmax(logits, k, renormalize=False)
+    return x, w1, w2, tw, ids
+
+
+def test_reference_case(dev):
+    # test_fused_moe.py:154-259: seq 128, in 128, hidden 256 (I = 128), out 128, 4 experts, top-2,
+    # fp16, renormalize=True, tolerance atol = rtol = 1e-3 ... on out_size = 128 columns; the
+    # reference allows w2 [E, out, I] with out != in; here H is shared by both GEMMs
+    from dlcompiler_amd.kernels.fused_moe import fused_moe
+
+    x, w1, w2, tw, ids = _inputs(128, 128, 128, 4, 2, 0, torch.float16, uniform=True)
+    out = fused_moe(x.to(dev), w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev), topk=2,
+                    renormalize=True).cpu()
+    ref = ofm.fused_moe(x, w1, w2, tw, ids, renormalize=True)
+    torch.testing.assert_close(out, ref, atol=1e-3, rtol=1e-3)
+
+
+@pytest.mark.parametrize("T,H,I,E,k", [(256, 256, 128, 8, 2), (1, 128, 128, 4, 1),
+                                       (333, 512, 384, 64, 6), (512, 2048, 1408, 8, 6)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_moe_parity(dev, T, H, I, E, k, dtype):
+    from dlcompiler_amd.kernels.fused_moe import fused_moe, shuffle_moe_weight
+
+    x, w1, w2, tw, ids = _inputs(T, H, I, E, k, 1, dtype)
+    args = (x.to(dev), w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev))
+    out = fused_moe(*args, k, renormalize=True)
+    ref = ofm.fused_moe(x, w1, w2, tw, ids, renormalize=True)
+    assert out.shape == (T, H) and out.dtype == dtype
+    # north-star tolerance for 16-bit outputs: 2e-2 abs/rel, the absolute part taken relative
+    # to the output scale (a slot value's 16-bit rounding is proportional to its magnitude)
+    scale = max(1.0, ref.float().abs().max().item())
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2 * scale)
+    err = ((out.cpu().double() - ref.double()).norm() / ref.double().norm()).item()
+    assert err < 5e-3
+    out2 = fused_moe(args[0], shuffle_moe_weight(args[1]), shuffle_moe_weight(args[2]), args[3],
+                     args[4], k, renormalize=True, weights_shuffled=True)
+    assert torch.equal(out2, out)
+
+
+def test_expert_shard(dev):
+    from dlcompiler_amd.kernels.fused_moe import fused_moe
+
+    x, w1, w2, tw, ids = _inputs(200, 256, 128, 8, 2, 2, torch.bfloat16)
+    d = lambda t: t.to(dev)
+    full = fused_moe(d(x), d(w1), d(w2), d(tw), d(ids), 2).cpu().float()
+    parts = [fused_moe(d(x), d(w1[o:o + 4].contiguous()), d(w2[o:o + 4].contiguous()), d(tw), d(ids),
+                       2, expert_offset=o, num_experts=8).cpu().float() for o in (0, 4)]
+    ref = ofm.fused_moe(x, w1[4:], w2[4:], tw, ids, expert_offset=4).float()
+    torch.testing.assert_close(parts[1], ref, rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(parts[0] + parts[1], full, rtol=2e-2, atol=2e-2)
+
+
+def test_get_start_end(dev):
+    # same values as the reference's docstring identity (fused_moe.py:271-275)
+    from dlcompiler_amd.kernels.fused_moe import get_start_end
+
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, 16, (300, 4), generator=g)
+    flat = ids.flatten().to(dev)
+    sorted_idx = flat.argsort()
+    start, end = get_start_end(flat, sorted_idx, 16)
+    rs, re_ = og.start_end(ids, 16)
+    assert start.dtype == sorted_idx.dtype
+    assert torch.equal(start.cpu(), rs) and torch.equal(end.cpu(), re_)
