@@ -44,51 +44,81 @@ __global__ __launch_bounds__(kThreads) void align_count_kernel(const int32_t* __
   for (int e = threadIdx.x; e < E; e += kThreads) chunk_counts[(int64_t)blockIdx.x * E + e] = hist[e];
 }
 
-// One workgroup of kMaxE threads; thread e owns expert e.
-__global__ __launch_bounds__(kMaxE) void align_scan_kernel(
+// One workgroup of 1024 threads: sub-group q = tid / E' (E' = E rounded up to 64) scans a
+// slice of the chunk rows for expert tid % E', the slices are combined through LDS, so the
+// dependent chain per thread is chunks / groups long instead of chunks.
+constexpr int kScanThreads = 1024;
+
+__global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
     int32_t* __restrict__ chunk_counts /* in: counts, out: start offsets */, int64_t chunks, int E,
     int block, int32_t numel, int32_t* __restrict__ sorted_ids, int64_t sorted_cap,
     int32_t* __restrict__ expert_ids, int64_t expert_ids_cap, int32_t* __restrict__ counts,
     int32_t* __restrict__ num_post_pad) {
-  __shared__ int32_t padded_s[kMaxE];
+  __shared__ int32_t part_s[kScanThreads];  // [group][expert'] slice totals -> slice bases
+  __shared__ int32_t total_s[kMaxE];
   __shared__ int32_t base_s[kMaxE + 1];
-  const int e = threadIdx.x;
-  int32_t total = 0;
-  if (e < E) {
-    for (int64_t c = 0; c < chunks; ++c) total += chunk_counts[c * E + e];
-  }
-  const int32_t padded = (e < E) ? (int32_t)(ceil_div(total, block) * block) : 0;
-  padded_s[e] = padded;
+  const int tid = threadIdx.x;
+  const int ep = (E + 63) & ~63;           // experts rounded up to a whole wave
+  const int groups = kScanThreads / ep;     // >= 4 for E <= 256
+  const int e = tid % ep, q = tid / ep;
+  const bool live = (e < E) && (q < groups);
+  const int64_t per = (chunks + groups - 1) / groups;
+  const int64_t c0 = q * per, c1 = (c0 + per < chunks) ? c0 + per : chunks;
+
+  int32_t slice = 0;
+  if (live)
+    for (int64_t c = c0; c < c1; ++c) slice += chunk_counts[c * E + e];
+  part_s[tid] = slice;
   __syncthreads();
-  if (e == 0) {
+  if (tid < E) {  // exclusive scan over the groups of this expert, total
     int32_t run = 0;
-    for (int i = 0; i < E; ++i) {
-      base_s[i] = run;
-      run += padded_s[i];
+    for (int g2 = 0; g2 < groups; ++g2) {
+      const int32_t v = part_s[g2 * ep + tid];
+      part_s[g2 * ep + tid] = run;
+      run += v;
     }
-    base_s[E] = run;
-    *num_post_pad = run;
+    total_s[tid] = run;
+  }
+  __syncthreads();
+  if (tid < 64) {  // padded totals -> expert bases: wave scan over up to 256 experts
+    int32_t run = 0;
+    for (int i0 = 0; i0 < E; i0 += 64) {
+      const int i = i0 + tid;
+      const int32_t padded = (i < E) ? (int32_t)(ceil_div(total_s[i], block) * block) : 0;
+      int32_t incl = padded;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d);
+        if (tid >= d) incl += up;
+      }
+      if (i < E) base_s[i] = run + incl - padded;
+      run += __shfl(incl, 63);
+    }
+    if (tid == 0) {
+      base_s[E] = run;
+      *num_post_pad = run;
+    }
   }
   __syncthreads();
   const int32_t total_padded = base_s[E];
-  if (e < E) {
-    const int32_t base = base_s[e];
-    if (counts) counts[e] = total;
-    // chunk start offsets for the placement pass
-    int32_t run = base;
-    for (int64_t c = 0; c < chunks; ++c) {
+  if (live) {
+    // chunk start offsets of this slice for the placement pass
+    int32_t run = base_s[e] + part_s[q * ep + e];
+    for (int64_t c = c0; c < c1; ++c) {
       const int32_t n = chunk_counts[c * E + e];
       chunk_counts[c * E + e] = run;
       run += n;
     }
-    // pad slots of this expert
-    for (int32_t p = base + total; p < base + padded; ++p) sorted_ids[p] = numel;
-    // block -> expert
-    for (int32_t b = base / block; b < (base + padded) / block; ++b) expert_ids[b] = e;
+  }
+  if (tid < E) {
+    const int32_t base = base_s[tid], total = total_s[tid], next = base_s[tid + 1];
+    if (counts) counts[tid] = total;
+    for (int32_t p = base + total; p < next; ++p) sorted_ids[p] = numel;   // pad slots
+    for (int32_t b = base / block; b < next / block; ++b) expert_ids[b] = tid;
   }
   // tails beyond the padded total
-  for (int64_t p = (int64_t)total_padded + e; p < sorted_cap; p += kMaxE) sorted_ids[p] = numel;
-  for (int64_t b = (int64_t)total_padded / block + e; b < expert_ids_cap; b += kMaxE)
+  for (int64_t p = (int64_t)total_padded + tid; p < sorted_cap; p += kScanThreads) sorted_ids[p] = numel;
+  for (int64_t b = (int64_t)total_padded / block + tid; b < expert_ids_cap; b += kScanThreads)
     expert_ids[b] = -1;
 }
 
@@ -173,7 +203,7 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
   int32_t* chunk_counts = (int32_t*)ws;
   hipLaunchKernelGGL(align_count_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
                      numel, E, chunk_counts);
-  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kMaxE), 0, s, chunk_counts, chunks, E, block,
+  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, chunk_counts, chunks, E, block,
                      (int32_t)numel, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, counts,
                      num_post_pad);
   if (numel > 0)
