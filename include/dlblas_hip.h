@@ -214,6 +214,47 @@ int dlb_moe_gemm_16bit_down(const void* act, const void* w2, const int32_t* sort
                             int expert_offset, int num_local_experts, int w_layout, void* out,
                             int dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Decoder-layer helpers around the attention / MoE kernels (memory-bound).
+ * ---------------------------------------------------------------------------------------- */
+
+/* fill_kv_cache: scatter the new K/V tokens of each sequence into the paged cache.
+ * Replaces fill_kv_cache + _fill_kv_cache_kernel, kernels/fill_kv_cache.py:23-185.
+ *   k_states/v_states [num_tokens, heads, head_dim(_v)]  (token / head strides, unit last)
+ *   k_cache/v_cache   [pages, page, heads, head_dim(_v)] (page / slot / head strides)
+ *   sequence b owns tokens q_start_loc[b] .. + q_seq_len[b]; its i-th new token lands at
+ *   context position kv_seq_len[b] - q_seq_len[b] + i, i.e. page
+ *   block_table[b][pos / page], slot pos % page.  Tokens outside every sequence are ignored.
+ * elem_size = bytes per element (the copy is type-agnostic); strides in elements. */
+int dlb_fill_kv_cache(const void* k_states, const void* v_states, void* k_cache, void* v_cache,
+                      const int32_t* q_start_loc, const int32_t* q_seq_len,
+                      const int32_t* kv_seq_len, const int32_t* block_table, int64_t num_tokens,
+                      int batch, int heads, int head_dim, int head_dim_v, int page, int max_blocks,
+                      int elem_size, int64_t ks_stride_tok, int64_t ks_stride_head,
+                      int64_t vs_stride_tok, int64_t vs_stride_head, int64_t kc_stride_page,
+                      int64_t kc_stride_slot, int64_t kc_stride_head, int64_t vc_stride_page,
+                      int64_t vc_stride_slot, int64_t vc_stride_head, int64_t bt_stride,
+                      void* stream);
+
+/* rms_norm: out = weight * round(x * rsqrt(mean(x^2) + eps)); with `residual` != NULL the
+ * input is first replaced by round(x + residual), which is also written to out_residual.
+ * Replaces rms_norm / add_rms_norm, kernels/rms_norm.py:8-133 and kernels/add_rms_norm.py:9-80.
+ * x/out/residual/out_residual [M, N] with row strides, weight [N]; bf16/f16, N % 8 == 0,
+ * N <= 16384. */
+int dlb_rms_norm(const void* x, const void* weight, const void* residual, void* out,
+                 void* out_residual, int64_t M, int N, int64_t ld_x, int64_t ld_res,
+                 int64_t ld_out, int64_t ld_out_res, float eps, int dtype, void* stream);
+
+/* apply_rotary_pos_emb: out = x * cos + rotate_half(x) * sin on q [T, Hq, D] and k [T, Hk, D],
+ * cos/sin [T, D] (row stride cs_stride_tok); outputs may alias the inputs.
+ * Replaces apply_rotary_pos_emb, kernels/apply_rotary_pos_emb.py:8-164.  bf16/f16, D % 16 == 0. */
+int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void* cos, const void* sin,
+                             void* q_out, void* k_out, int64_t num_tokens, int Hq, int Hk, int D,
+                             int64_t q_stride_tok, int64_t q_stride_head, int64_t k_stride_tok,
+                             int64_t k_stride_head, int64_t qo_stride_tok, int64_t qo_stride_head,
+                             int64_t ko_stride_tok, int64_t ko_stride_head, int64_t cs_stride_tok,
+                             int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
