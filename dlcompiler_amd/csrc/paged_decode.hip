@@ -44,6 +44,9 @@ struct DecodeParams {
   int max_blocks;
   int keys_per_split, nsplit_max;
   float scale_log2e;
+  float sm_scale;
+  int window;      // > 0: keys older than (ctx - 1 - window) are masked (paged_attention.py:163-167)
+  float softcap;   // > 0: logits -> softcap * tanh(logits / softcap) (paged_attention.py:186-189)
 };
 
 template <int DT>
@@ -94,9 +97,12 @@ __global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const Deco
   const int hchunk = unit - kvh * p.hchunks;
   const int b = blockIdx.z;
   const int ctx = p.kv_len[b];
-  const int k_begin = split * p.keys_per_split;
+  const int kv_min = p.window > 0 ? max(ctx - 1 - p.window, 0) : 0;  // first visible key
+  int k_begin = split * p.keys_per_split;
   if (k_begin >= ctx) return;  // uniform for the wave; also covers ctx <= 0
   const int k_end = min(ctx, k_begin + p.keys_per_split);
+  if (k_end <= kv_min) return;  // chunk entirely outside the sliding window
+  k_begin = max(k_begin, kv_min & ~(kTile - 1));  // start at the tile that holds kv_min
 
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;  // lane group 0..3
@@ -216,7 +222,10 @@ __global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const Deco
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = t0 + 16 * sub + 4 * g + i;
-        const float x = (key < k_end) ? s[sub][i] * p.scale_log2e : -__builtin_inff();
+        float x = s[sub][i] * p.scale_log2e;
+        if (p.softcap > 0.0f)
+          x = p.softcap * tanhf(s[sub][i] * p.sm_scale / p.softcap) * 1.4426950408889634f;
+        x = (key < k_end && key >= kv_min) ? x : -__builtin_inff();
         s[sub][i] = x;
         mloc = fmaxf(mloc, x);
       }
@@ -288,11 +297,13 @@ __global__ __launch_bounds__(D) void paged_decode_combine_kernel(const DecodePar
   float acc = 0.0f;
   if (ctx > 0) {
     const int ns = (ctx + p.keys_per_split - 1) / p.keys_per_split;
+    // chunks entirely before the sliding window were skipped by the split kernel
+    const int s0 = p.window > 0 ? max(ctx - 1 - p.window, 0) / p.keys_per_split : 0;
     const int64_t slot0 = ((int64_t)b * p.Hq + head) * p.nsplit_max;
     float m = -__builtin_inff();
-    for (int s = 0; s < ns; ++s) m = fmaxf(m, p.ws_ml[(slot0 + s) * 2]);
+    for (int s = s0; s < ns; ++s) m = fmaxf(m, p.ws_ml[(slot0 + s) * 2]);
     float den = 0.0f;
-    for (int s = 0; s < ns; ++s) {
+    for (int s = s0; s < ns; ++s) {
       const float w = __builtin_amdgcn_exp2f(p.ws_ml[(slot0 + s) * 2] - m);
       den += w * p.ws_ml[(slot0 + s) * 2 + 1];
       acc += w * p.ws_o[(slot0 + s) * D + d];
@@ -340,7 +351,8 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
                                      int64_t k_stride_tok, int64_t k_stride_head,
                                      int64_t v_stride_page, int64_t v_stride_tok,
                                      int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
-                                     int64_t bt_stride, float sm_scale, int dtype, void* ws,
+                                     int64_t bt_stride, float sm_scale, int window_size,
+                                     float logit_softcapping, int dtype, void* ws,
                                      size_t ws_bytes, void* stream) {
   using namespace dlb;
   if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || page < 1 || max_blocks < 1) return DLB_ERR_BAD_ARG;
@@ -395,6 +407,9 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   p.keys_per_split = pick_keys_per_split(B, Hkv, p.hchunks, max_ctx);
   p.nsplit_max = (max_ctx + p.keys_per_split - 1) / p.keys_per_split;
   p.scale_log2e = sm_scale * 1.4426950408889634f;
+  p.sm_scale = sm_scale;
+  p.window = window_size;
+  p.softcap = logit_softcapping;
   p.ws_o = (float*)ws;
   p.ws_ml = p.ws_o + (size_t)B * Hq * p.nsplit_max * D;
 

@@ -32,13 +32,13 @@ def paged_attention_fwd(
     [pages, page_size, Hkv, D]; ``block_offsets`` [batch, max_blocks] maps a sequence's
     logical pages to physical ones; ``kv_seqlens`` [batch] context lengths.  The decode case
     (one query token per sequence, ``q.shape[-3] == q_seqlens.size(0)``,
-    paged_attention.py:559) is implemented; sliding window and logit soft-capping are not.
+    paged_attention.py:559) is implemented, including the sliding window and logit soft-capping.
     """
     _lib.require_cuda(q, k, v, o, block_offsets, kv_seqlens)
-    if window_size is not None and window_size > 0:
-        raise NotImplementedError("sliding-window paged attention is not implemented")
-    if logit_softcapping is not None and logit_softcapping > 0:
-        raise NotImplementedError("logit soft-capping is not implemented")
+    if window_size is None:
+        window_size = -1
+    if logit_softcapping is None:
+        logit_softcapping = -1.0
     Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
     assert Lq == Lk, Lv == o.shape[-1]
     if sm_scale is None:
@@ -76,6 +76,7 @@ def paged_attention_fwd(
             kv_seqlens.data_ptr(), batch, head, num_kv_heads, Lq, page, max_blocks,
             q3.stride(0), q3.stride(1), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), o3.stride(0), o3.stride(1),
-            block_offsets.stride(0), float(sm_scale), _lib.torch_dtype_code(q.dtype),
+            block_offsets.stride(0), float(sm_scale), int(window_size), float(logit_softcapping),
+            _lib.torch_dtype_code(q.dtype),
             ws.data_ptr(), ws.numel(), _lib.current_stream_ptr(q.device))
     _lib.check(st, "dlb_paged_decode_attn")

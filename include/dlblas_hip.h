@@ -101,6 +101,9 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
  *   kv_len       int32 [B]             context length; rows with kv_len <= 0 produce zeros
  * out[b, h] = softmax(q[b, h] . K[b, h / (Hq/Hkv)]^T * sm_scale) V, softmax in fp32 and P
  * rounded to `dtype` before P.V, as in the reference.
+ * window_size > 0 masks keys older than kv_len - 1 - window_size (sliding window,
+ * paged_attention.py:163-167,191-199); logit_softcapping > 0 replaces the scaled logits by
+ * cap * tanh(logits / cap) (:186-189); pass <= 0 to disable either.
  * Supported: dtype bf16/f16, D in {64, 128}, page % 16 == 0, all strides multiples of 8 and
  * base pointers 16-byte aligned.  ws: dlb_paged_decode_ws_bytes(...) bytes of device scratch
  * (split-KV partials), caller-owned.
@@ -112,8 +115,9 @@ int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cach
                           int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_tok,
                           int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_tok,
                           int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
-                          int64_t bt_stride, float sm_scale, int dtype, void* ws,
-                          size_t ws_bytes, void* stream);
+                          int64_t bt_stride, float sm_scale, int window_size,
+                          float logit_softcapping, int dtype, void* ws, size_t ws_bytes,
+                          void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Varlen causal flash-attention prefill on packed sequences, GQA.

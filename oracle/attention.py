@@ -21,17 +21,26 @@ import math
 import torch
 
 
-def _dense_attention(q, k, v, scale, causal):
-    """q [Hq, Lq, D], k/v [Hkv, Lk, D] -> [Hq, Lq, D] in q.dtype."""
+def _dense_attention(q, k, v, scale, causal, window=None, softcap=None):
+    """q [Hq, Lq, D], k/v [Hkv, Lk, D] -> [Hq, Lq, D] in q.dtype.  The queries are the last
+    Lq positions of the Lk keys.  ``window`` > 0 hides keys more than ``window`` positions
+    behind a query (python/dlBLAS/dlblas/kernels/paged_attention.py:163-167,191-199);
+    ``softcap`` > 0 maps the scaled scores to cap * tanh(scores / cap) (:186-189)."""
     hq, hkv = q.shape[0], k.shape[0]
     group = hq // hkv
     kk = k.float().repeat_interleave(group, dim=0)
     vv = v.float().repeat_interleave(group, dim=0)
     scores = torch.matmul(q.float(), kk.transpose(1, 2)) * scale
+    if softcap is not None and softcap > 0:
+        scores = torch.tanh(scores / softcap) * softcap
+    lq, lk = q.shape[1], k.shape[1]
     if causal:
-        lq, lk = q.shape[1], k.shape[1]
         keep = torch.ones(lq, lk, dtype=torch.bool).tril(diagonal=lk - lq)
         scores = scores.masked_fill(~keep, float("-inf"))
+    if window is not None and window > 0:
+        qpos = torch.arange(lk - lq, lk)[:, None]
+        far = torch.arange(lk)[None, :] < qpos - window
+        scores = scores.masked_fill(far, float("-inf"))
     p = torch.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
     return torch.matmul(p.float(), vv).to(q.dtype)
 
@@ -58,7 +67,8 @@ def gather_paged(cache, block_table_row, length):
     return pages.reshape(n * page, *cache.shape[2:])[:length]
 
 
-def paged_decode(q, k_cache, v_cache, block_table, kv_len, sm_scale=None):
+def paged_decode(q, k_cache, v_cache, block_table, kv_len, sm_scale=None, window=None,
+                 softcap=None):
     """q [B, Hq, D] -> o [B, Hq, D]; sequences with kv_len <= 0 give zeros."""
     scale = sm_scale if sm_scale is not None else 1.0 / math.sqrt(q.shape[-1])
     o = torch.zeros_like(q)
@@ -67,7 +77,7 @@ def paged_decode(q, k_cache, v_cache, block_table, kv_len, sm_scale=None):
             continue
         kk = gather_paged(k_cache, block_table[b], length).transpose(0, 1)
         vv = gather_paged(v_cache, block_table[b], length).transpose(0, 1)
-        o[b] = _dense_attention(q[b][:, None, :], kk, vv, scale, False)[:, 0, :]
+        o[b] = _dense_attention(q[b][:, None, :], kk, vv, scale, False, window, softcap)[:, 0, :]
     return o
 
 

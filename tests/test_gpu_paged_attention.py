@@ -12,7 +12,7 @@ def _rand(shape, seed, dtype):
 
 
 def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_dtype=torch.int32,
-              sm_scale=None, uniform=False):
+              sm_scale=None, uniform=False, window=None, softcap=None):
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
     if uniform:   # the reference test draws torch.rand inputs (test_paged_attention.py:157-180)
@@ -26,11 +26,12 @@ def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_
     q = mk((B, hq, d), 7)
     kc, vc, table = oa.make_paged_cache(ks, vs, page, num_pages=num_pages, seed=seed, dtype=dtype)
     kv_len = torch.tensor(lens)
-    ref = oa.paged_decode(q, kc, vc, table, kv_len, sm_scale=sm_scale)
+    ref = oa.paged_decode(q, kc, vc, table, kv_len, sm_scale=sm_scale, window=window, softcap=softcap)
     o = torch.full((B, hq, d), 9.0, dtype=dtype, device=dev)
     ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(table_dtype).to(dev),
                               torch.arange(B, device=dev), torch.ones(B, dtype=torch.int64, device=dev),
-                              kv_len.to(dev), 1, sm_scale=sm_scale)
+                              kv_len.to(dev), 1, sm_scale=sm_scale, window_size=window,
+                              logit_softcapping=softcap)
     assert ret is None
     out = o.cpu()
     assert torch.isfinite(out.float()).all()              # NaN-filled unused cache never read
@@ -61,6 +62,21 @@ def test_context_length_edges(dev, dtype, page):
 def test_group_sizes_and_scale(dev):
     for hq, hkv in [(8, 8), (16, 2), (32, 1), (40, 2)]:
         _run_case(dev, [300, 77, 1025], hq, hkv, 64, 32, torch.bfloat16, sm_scale=0.2)
+
+
+# the reference's window case uses win_size 32 on the same sequences (test_paged_attention.py:
+# 288-346, ground truth from flash_attn which is not available here; the oracle restates the
+# kernel's own mask, paged_attention.py:163-167,191-199)
+@pytest.mark.parametrize("window", [32, 1, 600, 5000])
+def test_sliding_window(dev, window):
+    _run_case(dev, [51, 41, 31, 21, 1, 700, 2049], 8, 2, 128, 16, torch.float16, window=window)
+    _run_case(dev, [513, 1200, 64], 32, 8, 128, 64, torch.bfloat16, window=window)
+
+
+@pytest.mark.parametrize("cap", [30.0, 5.0, 0.5])
+def test_logit_softcapping(dev, cap):
+    _run_case(dev, [300, 77, 1025, 1], 16, 4, 128, 64, torch.bfloat16, softcap=cap)
+    _run_case(dev, [300, 2000], 8, 2, 64, 16, torch.float16, softcap=cap, window=100)
 
 
 def test_non_power_of_two_page_and_spare_pages(dev):
@@ -102,8 +118,6 @@ def test_unsupported_requests_raise(dev):
             torch.ones(2, device=dev), torch.tensor([3, 4], device=dev), 1)
     with pytest.raises(RuntimeError):
         paged_attention_fwd(*args)                           # head dim 48
-    with pytest.raises(NotImplementedError):
-        paged_attention_fwd(*args, window_size=32)
 
 
 def test_config4_full(dev):

@@ -82,3 +82,22 @@ def test_paged_decode_zero_length_and_scale():
     a = oa.paged_decode(q, kc, vc, table, torch.tensor([20]), sm_scale=0.0)
     torch.testing.assert_close(a[0, 0].float(), vs[0][:, 0].float().mean(0), rtol=2e-2, atol=2e-2)
     assert math.isfinite(a.float().sum().item())
+
+
+def test_window_and_softcap_closed_forms():
+    ks, vs = [_rand((50, 1, 16), 1)], [_rand((50, 1, 16), 2)]
+    kc, vc, table = oa.make_paged_cache(ks, vs, page=16)
+    q = _rand((1, 2, 16), 3)
+    n = torch.tensor([50])
+    base = oa.paged_decode(q, kc, vc, table, n)
+    assert torch.equal(oa.paged_decode(q, kc, vc, table, n, window=49), base)      # window covers all
+    assert torch.equal(oa.paged_decode(q, kc, vc, table, n, window=1000), base)
+    # the window keeps the current token and `window` older ones: same as a shorter context
+    short = oa.make_paged_cache([ks[0][39:]], [vs[0][39:]], page=16)
+    assert torch.equal(oa.paged_decode(q, kc, vc, table, n, window=10),
+                       oa.paged_decode(q, short[0], short[1], short[2], torch.tensor([11])))
+    # soft cap: huge cap is the identity, tiny cap flattens the logits -> mean of V
+    torch.testing.assert_close(oa.paged_decode(q, kc, vc, table, n, softcap=1e6).float(), base.float(),
+                               rtol=1e-2, atol=1e-2)
+    flat = oa.paged_decode(q, kc, vc, table, n, softcap=1e-4)
+    torch.testing.assert_close(flat[0, 0].float(), vs[0][:, 0].float().mean(0), rtol=2e-2, atol=2e-2)
