@@ -33,6 +33,8 @@ SIGNATURES = {
                               + [c_float, c_int, c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "dlb_prefill_attn_varlen": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 8
                                 + [c_float, c_int, c_void_p]),
+    "dlb_paged_prefill_attn": (c_int, [c_void_p] * 8 + [c_int] * 7 + [c_int64] * 11
+                               + [c_float, c_int, c_float, c_int, c_void_p]),
     "dlb_per_token_group_quant_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                               c_int64, c_int64, c_int64, c_int, c_void_p]),
     "dlb_moe_gemm_fp8_gate_up": (c_int, [c_void_p] * 6 + [c_int] * 9 + [c_void_p] * 3),

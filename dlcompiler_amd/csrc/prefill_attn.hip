@@ -34,6 +34,16 @@ struct PrefillParams {
   int Hq, Hkv, group;
   int xcd_heads;  // != 0: remap blockIdx.x so the heads of a KV group share an XCD
   float scale_log2e;
+  // paged K/V (PAGED kernels): k/v point at caches [pages, page, Hkv, D]; *_st is the slot
+  // stride, *_sp the page stride; sequence s reads pages block_table[s][.] and its queries sit
+  // at context positions kv_len[s] - seq_len[s] + i
+  const int32_t* kv_len;
+  const int32_t* block_table;
+  int64_t bt_stride, k_sp, v_sp;
+  int page, page_shift;
+  // generic masking (both layouts): sliding window (> 0) and logit soft-cap (> 0)
+  int window;
+  float softcap, sm_scale;
 };
 
 template <int DT>
@@ -81,7 +91,7 @@ struct Smem {
 #ifndef DLB_PF_OCC
 #define DLB_PF_OCC 2
 #endif
-template <int DT, int D>
+template <int DT, int D, bool PAGED>
 __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int KS = D / 16;  // MFMA k-steps over the head dim for S^T
   constexpr int MT = D / 32;  // 32-row tiles of O^T
@@ -98,6 +108,10 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   const int q0 = qtile * kBlockM;
   if (q0 >= L) return;
   const int64_t tok0 = p.start_loc[seq];
+  // context seen by this sequence: kv_total keys, the queries are its last L positions
+  const int kv_total = PAGED ? p.kv_len[seq] : L;
+  const int hist = kv_total - L;
+  if (PAGED && hist < 0) return;  // inconsistent lengths: nothing sensible to compute
   int head = blockIdx.x;
   if (p.xcd_heads) head = (blockIdx.x & 7) * (p.Hq >> 3) + (blockIdx.x >> 3);
   const int kvh = head / p.group;
@@ -122,12 +136,20 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qp + 16 * ks);
   }
 
-  const int kv_end = min(L, q0 + kBlockM);            // keys this workgroup needs
+  const int kv_end = min(kv_total, hist + q0 + kBlockM);  // keys this workgroup needs
   const int ntiles = (kv_end + kTileN - 1) / kTileN;
+  // window / soft-cap requests take the masked path for every tile
+  // (only the paged entry point exposes them; the packed kernel compiles them out)
+  const int window = PAGED ? p.window : -1;
+  const float softcap = PAGED ? p.softcap : -1.0f;
+  const bool generic = (window > 0) || (softcap > 0.0f);
   // tiles below this index lie entirely under the diagonal for every wave of the workgroup
-  // (q0 is a multiple of 128): no mask, no clamping of key rows
-  const int nfull = q0 / kTileN;
-  const int wave_last_row = q0 + 32 * wave + 31;
+  // (all 64 keys <= position of row q0): no mask, no clamping of key rows
+  const int nfull = generic ? 0 : (hist + q0 + 1) / kTileN;
+  // first tile that can hold a visible key (sliding window)
+  const int jfirst = window > 0 ? max(hist + q0 - window, 0) / kTileN : 0;
+  const int qpos = hist + qrow;                          // context position of this lane's query
+  const int wave_last_pos = hist + q0 + 32 * wave + 31;
 
   // ---- global -> register staging of one K/V tile.  Per-thread base pointers are formed
   // once; a tile adds a workgroup-uniform offset.  CLAMP (tiles that may run past the
@@ -141,8 +163,24 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   const int k_lrow = lane / DG;                   // row inside an instruction
   const int k_pos = lane % DG;                    // 16-byte position inside the row
   const unsigned char* kbytes = (const unsigned char*)kb;
-  const unsigned char* vbase = (const unsigned char*)vb + ((tok0 + 4 * (tid / DG)) * p.v_st + 8 * (tid % DG)) * 2;
+  const unsigned char* vbytes = (const unsigned char*)vb + 16 * (tid % DG);
   const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
+  const int32_t* bt = PAGED ? p.block_table + (int64_t)seq * p.bt_stride : nullptr;
+  // byte address of key row `key` of this sequence (page lookup for the paged layout)
+  auto k_row = [&](int key) -> const unsigned char* {
+    if (PAGED) {
+      const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
+      return kbytes + ((int64_t)bt[pi] * p.k_sp + (int64_t)(key - pi * p.page) * p.k_st) * 2;
+    }
+    return kbytes + (tok0 + key) * k_row_bytes;
+  };
+  auto v_row = [&](int key) -> const unsigned char* {
+    if (PAGED) {
+      const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
+      return vbytes + ((int64_t)bt[pi] * p.v_sp + (int64_t)(key - pi * p.page) * p.v_st) * 2;
+    }
+    return vbytes + (tok0 + key) * v_row_bytes;
+  };
   const bool v_active = (VUNITS >= kThreads) || (tid < VUNITS);
   u32x4 vreg[4];
   static_assert(VLD == 1, "one (4 keys x 8 dims) V unit per thread");
@@ -154,18 +192,20 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
       const int q = 4 * i + wave;                 // which 1 KB slice of the tile
       const int r = q * KRPI + k_lrow;            // key row inside the tile
       int key = t0 + r;
-      if (CLAMP) key = min(key, L - 1);
-      const unsigned char* src = kbytes + (tok0 + key) * k_row_bytes + ((k_pos ^ (r & (DG - 1))) << 4);
+      if (CLAMP) key = min(key, kv_total - 1);
+      const unsigned char* src = k_row(key) + ((k_pos ^ (r & (DG - 1))) << 4);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (__attribute__((address_space(3))) void*)(ks + q * 1024),
                                        16, 0, 0);
     }
     if (v_active) {
+      // the 4 keys of a unit share a page (page % 4 == 0)
+      const int key0 = t0 + 4 * (tid / DG);
+      const unsigned char* v0 = v_row(CLAMP ? min(key0, kv_total - 1) : key0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        int row = t0 + r;  // + 4 * (tid / DG) is in vbase
-        if (CLAMP) row = min(row + 4 * (tid / DG), L - 1) - 4 * (tid / DG);
-        vreg[r] = *(const u32x4*)(vbase + row * v_row_bytes);
+        const int rr = CLAMP ? max(min(r, kv_total - 1 - key0), 0) : r;
+        vreg[r] = *(const u32x4*)(v0 + rr * v_row_bytes);
       }
     }
   };
@@ -210,7 +250,8 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   auto process_tile = [&](auto mask_tag, int j) {
     constexpr bool MASK = decltype(mask_tag)::value;
     const int t0 = j * kTileN;
-    if (MASK && t0 > wave_last_row) return;  // wave-uniform: tile entirely above the diagonal
+    if (MASK && t0 > wave_last_pos) return;  // wave-uniform: tile entirely above the diagonal
+    if (MASK && window > 0 && t0 + kTileN - 1 < wave_last_pos - 31 - window) return;  // below the window
     const unsigned char* ks = smem + (j & 1) * SM::stage;
     const unsigned char* vs = ks + SM::kBytes;
 
@@ -238,7 +279,12 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
       for (int i = 0; i < 16; ++i) {
         if (MASK) {
           const int key = t0 + 32 * nt + 8 * (i >> 2) + 4 * hh + (i & 3);
-          s[nt][i] = (key <= qrow) ? s[nt][i] : -__builtin_inff();
+          float x = s[nt][i];
+          if (softcap > 0.0f)  // cap * tanh(x * scale / cap), kept in raw-score units
+            x = tanhf(x * (p.sm_scale / softcap)) * (softcap / p.sm_scale);
+          bool vis = key <= qpos;
+          if (window > 0) vis = vis && (key >= qpos - window);
+          s[nt][i] = vis ? x : -__builtin_inff();
         }
         mloc = fmaxf(mloc, s[nt][i]);
       }
@@ -246,7 +292,8 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * cs;
     if (__any(mloc > m_run + kRescaleGap)) {
       const float m_new = fmaxf(m_run, mloc);  // finite from tile 0 on (key 0 is visible)
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      // (a fully masked row under a sliding window keeps m_new = -inf: leave it untouched)
+      const float alpha = (MASK && PAGED && m_new == -__builtin_inff()) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -254,12 +301,14 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
     }
+    // a row whose keys so far were all masked (sliding window) still has m_run = -inf
+    const float m_ref = (MASK && PAGED && m_run == -__builtin_inff()) ? 0.0f : m_run;
     float psum = 0.0f;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][i], cs, -m_run));
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][i], cs, -m_ref));
         s[nt][i] = e;
         psum += e;
       }
@@ -293,12 +342,12 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   // vmcnt(0): the direct-to-LDS loads of this wave have landed before the barrier publishes
   // the buffer (encoding: vmcnt = 0, expcnt / lgkmcnt left at their maxima)
   auto wait_dma = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
-  if (nfull > 0) load_tile(NoClamp{}, 0, 0); else load_tile(Clamp{}, 0, 0);
-  store_tile(0);
+  int j = jfirst;
+  if (j < nfull) load_tile(NoClamp{}, j * kTileN, j & 1); else load_tile(Clamp{}, j * kTileN, j & 1);
+  store_tile(j & 1);
   wait_dma();
   __syncthreads();
 
-  int j = 0;
   // tiles under the diagonal whose successor is also under it: nothing to mask or clamp
   for (; j + 1 < nfull; ++j) {
     load_tile(NoClamp{}, (j + 1) * kTileN, (j + 1) & 1);
@@ -321,7 +370,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   // ---- epilogue: normalise and store O (lane holds 4 consecutive dims per register quad)
   l_run += __shfl_xor(l_run, 32);
   if (qrow < L) {
-    const float inv = 1.0f / l_run;
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
     unsigned short* op = (unsigned short*)p.o + (tok0 + qrow) * p.o_st + (int64_t)head * p.o_sh;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -334,6 +383,57 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
       }
     }
   }
+}
+
+}  // namespace
+}  // namespace dlb
+
+namespace dlb {
+namespace {
+
+// Shared argument checks and launch of both entry points; the paged fields of `p` are already
+// filled in (or zeroed) by the caller.
+int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int D, int max_len,
+                   float sm_scale, int dtype, void* stream) {
+  if (D != 64 && D != 128) return DLB_ERR_UNSUPPORTED;
+  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) ||
+      (reinterpret_cast<uintptr_t>(p.o) & 7u) != 0)
+    return DLB_ERR_UNSUPPORTED;
+  const int64_t in_strides[] = {p.q_st, p.q_sh, p.k_st, p.k_sh, p.v_st, p.v_sh, p.k_sp, p.v_sp};
+  for (int64_t sd : in_strides)
+    if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
+  if (p.o_st % 4 != 0 || p.o_sh % 4 != 0) return DLB_ERR_UNSUPPORTED;
+  if (B > 65535) return DLB_ERR_UNSUPPORTED;
+  if (!(sm_scale > 0.0f)) return DLB_ERR_BAD_ARG;  // the tile maximum is taken before scaling
+
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.group = Hq / Hkv;
+  // workgroups are dealt round-robin to the 8 XCDs by linear id; with Hq % 8 == 0 the
+  // remap in the kernel puts heads {x, x+8, ...} -> consecutive heads on one XCD so a KV
+  // group's four query heads hit the same L2.
+  p.xcd_heads = (Hq % 8 == 0 && Hq >= 16) ? 1 : 0;
+  p.scale_log2e = sm_scale * 1.4426950408889634f;
+  p.sm_scale = sm_scale;
+
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((uint32_t)Hq, (uint32_t)ceil_div(max_len, kBlockM), (uint32_t)B);
+  if (grid.y > 65535) return DLB_ERR_UNSUPPORTED;
+#define DLB_LAUNCH_PREFILL(DT_, D_, PG_) \
+  hipLaunchKernelGGL((prefill_attn_kernel<DT_, D_, PG_>), grid, dim3(kThreads), 0, s, p)
+#define DLB_DISPATCH_PREFILL(PG_)                              \
+  if (dtype == DLB_DTYPE_BF16) {                               \
+    if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 128, PG_); \
+    else DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 64, PG_);           \
+  } else {                                                     \
+    if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 128, PG_);  \
+    else DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 64, PG_);            \
+  }
+  if (paged) { DLB_DISPATCH_PREFILL(true) } else { DLB_DISPATCH_PREFILL(false) }
+#undef DLB_DISPATCH_PREFILL
+#undef DLB_LAUNCH_PREFILL
+  return launch_status();
 }
 
 }  // namespace
@@ -352,19 +452,7 @@ extern "C" int dlb_prefill_attn_varlen(const void* q, const void* k, const void*
   if (Hq % Hkv != 0) return DLB_ERR_BAD_ARG;
   if (B == 0 || max_len == 0) return DLB_OK;
   if (!q || !k || !v || !o || !start_loc || !seq_len) return DLB_ERR_BAD_ARG;
-  if (D != 64 && D != 128) return DLB_ERR_UNSUPPORTED;
-  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) ||
-      (reinterpret_cast<uintptr_t>(o) & 7u) != 0)
-    return DLB_ERR_UNSUPPORTED;
-  const int64_t in_strides[] = {q_stride_tok, q_stride_head, k_stride_tok,
-                                k_stride_head, v_stride_tok, v_stride_head};
-  for (int64_t sd : in_strides)
-    if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
-  if (o_stride_tok % 4 != 0 || o_stride_head % 4 != 0) return DLB_ERR_UNSUPPORTED;
-  if (B > 65535) return DLB_ERR_UNSUPPORTED;
-
-  PrefillParams p;
+  PrefillParams p = {};
   p.q = q;
   p.k = k;
   p.v = v;
@@ -379,27 +467,56 @@ extern "C" int dlb_prefill_attn_varlen(const void* q, const void* k, const void*
   p.v_sh = v_stride_head;
   p.o_st = o_stride_tok;
   p.o_sh = o_stride_head;
-  p.Hq = Hq;
-  p.Hkv = Hkv;
-  p.group = Hq / Hkv;
-  // workgroups are dealt round-robin to the 8 XCDs by linear id; with Hq % 8 == 0 the
-  // remap in the kernel puts heads {x, x+8, ...} -> consecutive heads on one XCD so a KV
-  // group's four query heads hit the same L2.
-  p.xcd_heads = (Hq % 8 == 0 && Hq >= 16) ? 1 : 0;
-  p.scale_log2e = sm_scale * 1.4426950408889634f;
+  p.page = 1;
+  p.page_shift = 0;
+  p.window = -1;
+  p.softcap = -1.0f;
+  return launch_prefill(p, false, B, Hq, Hkv, D, max_len, sm_scale, dtype, stream);
+}
 
-  hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((uint32_t)Hq, (uint32_t)ceil_div(max_len, kBlockM), (uint32_t)B);
-  if (grid.y > 65535) return DLB_ERR_UNSUPPORTED;
-#define DLB_LAUNCH_PREFILL(DT_, D_) \
-  hipLaunchKernelGGL((prefill_attn_kernel<DT_, D_>), grid, dim3(kThreads), 0, s, p)
-  if (dtype == DLB_DTYPE_BF16) {
-    if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 128);
-    else DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 64);
-  } else {
-    if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 128);
-    else DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 64);
-  }
-#undef DLB_LAUNCH_PREFILL
-  return launch_status();
+extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache,
+                                      void* o, const int32_t* block_table,
+                                      const int32_t* q_start_loc, const int32_t* q_len,
+                                      const int32_t* kv_len, int B, int Hq, int Hkv, int D,
+                                      int page, int max_blocks, int max_q_len,
+                                      int64_t q_stride_tok, int64_t q_stride_head,
+                                      int64_t k_stride_page, int64_t k_stride_tok,
+                                      int64_t k_stride_head, int64_t v_stride_page,
+                                      int64_t v_stride_tok, int64_t v_stride_head,
+                                      int64_t o_stride_tok, int64_t o_stride_head,
+                                      int64_t bt_stride, float sm_scale, int window_size,
+                                      float logit_softcapping, int dtype, void* stream) {
+  using namespace dlb;
+  if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || max_q_len < 0 || page < 1 || max_blocks < 0)
+    return DLB_ERR_BAD_ARG;
+  if (Hq % Hkv != 0) return DLB_ERR_BAD_ARG;
+  if (B == 0 || max_q_len == 0) return DLB_OK;
+  if (!q || !k_cache || !v_cache || !o || !block_table || !q_start_loc || !q_len || !kv_len)
+    return DLB_ERR_BAD_ARG;
+  if (page % 4 != 0) return DLB_ERR_UNSUPPORTED;  // a 4-key V unit must not straddle pages
+  PrefillParams p = {};
+  p.q = q;
+  p.k = k_cache;
+  p.v = v_cache;
+  p.o = o;
+  p.start_loc = q_start_loc;
+  p.seq_len = q_len;
+  p.kv_len = kv_len;
+  p.block_table = block_table;
+  p.bt_stride = bt_stride;
+  p.q_st = q_stride_tok;
+  p.q_sh = q_stride_head;
+  p.k_sp = k_stride_page;
+  p.k_st = k_stride_tok;
+  p.k_sh = k_stride_head;
+  p.v_sp = v_stride_page;
+  p.v_st = v_stride_tok;
+  p.v_sh = v_stride_head;
+  p.o_st = o_stride_tok;
+  p.o_sh = o_stride_head;
+  p.page = page;
+  p.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz((unsigned)page) : -1;
+  p.window = window_size;
+  p.softcap = logit_softcapping;
+  return launch_prefill(p, true, B, Hq, Hkv, D, max_q_len, sm_scale, dtype, stream);
 }

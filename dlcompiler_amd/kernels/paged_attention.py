@@ -30,9 +30,11 @@ def paged_attention_fwd(
 
     Args follow the reference: ``q`` [tokens, Hq, D]; ``k``/``v`` caches
     [pages, page_size, Hkv, D]; ``block_offsets`` [batch, max_blocks] maps a sequence's
-    logical pages to physical ones; ``kv_seqlens`` [batch] context lengths.  The decode case
-    (one query token per sequence, ``q.shape[-3] == q_seqlens.size(0)``,
-    paged_attention.py:559) is implemented, including the sliding window and logit soft-capping.
+    logical pages to physical ones; ``kv_seqlens`` [batch] context lengths.  One query token
+    per sequence (``q.shape[-3] == q_seqlens.size(0)``, paged_attention.py:559) takes the
+    split-KV decode kernel; anything else is the prefill-with-history case
+    (paged_attention.py:560-607): the last ``q_seqlens[s]`` context positions of sequence
+    ``s`` are its queries.  Sliding window and logit soft-capping apply to both.
     """
     _lib.require_cuda(q, k, v, o, block_offsets, kv_seqlens)
     if window_size is None:
@@ -45,9 +47,6 @@ def paged_attention_fwd(
         sm_scale = 1.0 / (Lq**0.5)
     batch, head = q_seqlens.shape[0], q.shape[-2]
     is_decoding = q.shape[-3] == q_seqlens.size(0)
-    if not is_decoding:
-        raise NotImplementedError(
-            "only the decode branch (one query token per sequence) is implemented")
     if Lv != Lk:
         raise NotImplementedError("value head size must equal key head size")
     assert k.dim() == 4 and v.dim() == 4 and k.shape[:3] == v.shape[:3]
@@ -58,16 +57,32 @@ def paged_attention_fwd(
     assert page >= 16
     for t in (q, k, v, o):
         assert t.stride(-1) == 1, "last dimension must be contiguous"
-    q3 = q.reshape(batch, head, Lq) if q.dim() != 3 else q
-    o3 = o.reshape(batch, head, Lv) if o.dim() != 3 else o
-    assert o3.data_ptr() == o.data_ptr()
     block_offsets = _as_int32(block_offsets)
     if block_offsets.stride(-1) != 1:
         block_offsets = block_offsets.contiguous()
     kv_seqlens = _as_int32(kv_seqlens).contiguous()
     max_blocks = block_offsets.size(1)
-
     lib = _lib.load()
+
+    if not is_decoding:
+        assert q.dim() == 3 and o.dim() == 3
+        q_start_loc = _as_int32(q_start_loc).contiguous()
+        q_seqlens = _as_int32(q_seqlens).contiguous()
+        with torch.cuda.device(q.device):
+            st = lib.dlb_paged_prefill_attn(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), block_offsets.data_ptr(),
+                q_start_loc.data_ptr(), q_seqlens.data_ptr(), kv_seqlens.data_ptr(), batch, head,
+                num_kv_heads, Lq, page, max_blocks, int(max_seqlen), q.stride(0), q.stride(1),
+                k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
+                o.stride(0), o.stride(1), block_offsets.stride(0), float(sm_scale),
+                int(window_size), float(logit_softcapping), _lib.torch_dtype_code(q.dtype),
+                _lib.current_stream_ptr(q.device))
+        _lib.check(st, "dlb_paged_prefill_attn")
+        return
+
+    q3 = q.reshape(batch, head, Lq) if q.dim() != 3 else q
+    o3 = o.reshape(batch, head, Lv) if o.dim() != 3 else o
+    assert o3.data_ptr() == o.data_ptr()
     ws_bytes = lib.dlb_paged_decode_ws_bytes(batch, head, num_kv_heads, Lq, page, max_blocks)
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):

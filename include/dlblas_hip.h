@@ -141,6 +141,32 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
                             int64_t o_stride_head, float sm_scale, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Causal attention of new query tokens over a paged KV cache that already holds them and
+ * their history (chunked prefill / prefix-cache hit), GQA.
+ * Replaces the non-decoding branch of paged_attention_fwd + _fwd_kernel,
+ * kernels/paged_attention.py:319-489, 559-607.
+ *   q [tokens, Hq, D], o [tokens, Hq, D]: sequence s owns query tokens q_start_loc[s] ..
+ *   q_start_loc[s] + q_len[s] - 1; k_cache/v_cache [pages, page, Hkv, D]; block_table int32
+ *   [B, max_blocks]; kv_len int32 [B] = history + q_len[s] (sequences with kv_len < q_len are
+ *   skipped).  Query i of sequence s sits at context position kv_len[s] - q_len[s] + i and
+ *   sees keys 0 .. that position (paged_attention.py:455), or, with window_size > 0, only the
+ *   keys >= position - window_size (:429-431,457-458); logit_softcapping > 0 replaces the
+ *   scaled logits by cap * tanh(logits / cap) (:450-453).  Pass <= 0 to disable either.
+ *   max_q_len >= max(q_len) sizes the grid.
+ * Supported: dtype bf16/f16, D in {64, 128}, page % 4 == 0, sm_scale > 0, q/k/v strides
+ * multiples of 8 and bases 16-byte aligned, o strides multiples of 4 and base 8-byte aligned.
+ * ---------------------------------------------------------------------------------------- */
+int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, void* o,
+                           const int32_t* block_table, const int32_t* q_start_loc,
+                           const int32_t* q_len, const int32_t* kv_len, int B, int Hq, int Hkv,
+                           int D, int page, int max_blocks, int max_q_len, int64_t q_stride_tok,
+                           int64_t q_stride_head, int64_t k_stride_page, int64_t k_stride_tok,
+                           int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_tok,
+                           int64_t v_stride_head, int64_t o_stride_tok, int64_t o_stride_head,
+                           int64_t bt_stride, float sm_scale, int window_size,
+                           float logit_softcapping, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * fp8 fused-MoE building blocks (OCP e4m3fn, fp32 scales per 128 along K; weights carry one
  * scale per 128 x 128 block).  Pipeline shape follows fused_moe, kernels/fused_moe.py:296-376
  * (grouped GEMM kernel :82-175); the fp8 scheme has no reference counterpart -- nearest

@@ -10,7 +10,12 @@
   (``_make_blocked_cache`` read backwards), then ``_naive_attention``: GQA expand,
   ``softmax(q k^T / sqrt(D))`` in fp32, cast to the query dtype, ``@ v``.
 
-Both evaluate the two matrix products with fp32 accumulation on the 16-bit inputs and do not
+* ``paged_prefill`` is the same ground truth for new tokens that follow a cached history
+  (test_paged_attention.py:15-27 ``_make_bias``: key j is hidden from query i when
+  ``j - i > history``), with the sliding window of ``_naive_window_attention`` (:87-113,
+  flash-attn ``window_size=(w, w)`` under ``causal=True``: keys ``>= position - w``).
+
+All evaluate the two matrix products with fp32 accumulation on the 16-bit inputs and do not
 round the scores to 16 bits (the reference's fp16 matmul on the device does); outputs are
 rounded once to the input dtype.
 """
@@ -78,6 +83,24 @@ def paged_decode(q, k_cache, v_cache, block_table, kv_len, sm_scale=None, window
         kk = gather_paged(k_cache, block_table[b], length).transpose(0, 1)
         vv = gather_paged(v_cache, block_table[b], length).transpose(0, 1)
         o[b] = _dense_attention(q[b][:, None, :], kk, vv, scale, False, window, softcap)[:, 0, :]
+    return o
+
+
+def paged_prefill(q, k_cache, v_cache, block_table, q_start_loc, q_len, kv_len, sm_scale=None,
+                  window=None, softcap=None):
+    """q [T, Hq, D] packed; sequence b owns rows q_start_loc[b] .. + q_len[b], which are the
+    last q_len[b] of its kv_len[b] cached positions.  Returns o [T, Hq, D]; rows outside any
+    sequence stay zero."""
+    scale = sm_scale if sm_scale is not None else 1.0 / math.sqrt(q.shape[-1])
+    o = torch.zeros_like(q)
+    for b, (start, lq, lk) in enumerate(zip(q_start_loc.tolist(), q_len.tolist(), kv_len.tolist())):
+        if lq <= 0 or lk < lq:
+            continue
+        kk = gather_paged(k_cache, block_table[b], lk).transpose(0, 1)
+        vv = gather_paged(v_cache, block_table[b], lk).transpose(0, 1)
+        sl = slice(start, start + lq)
+        o[sl] = _dense_attention(q[sl].transpose(0, 1), kk, vv, scale, True, window,
+                                 softcap).transpose(0, 1)
     return o
 
 

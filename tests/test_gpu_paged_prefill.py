@@ -1,0 +1,117 @@
+"""GPU parity: paged_attention_fwd, prefill-with-history branch, vs the CPU oracle through the
+C ABI."""
+import pytest
+import torch
+
+from oracle import attention as oa
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False, window=None,
+              softcap=None, sm_scale=None, max_seqlen=None, tol=2e-2):
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+
+    gen = torch.Generator().manual_seed(123 + seed)
+    if uniform:   # the reference test draws torch.rand inputs (test_paged_attention.py:157-180)
+        mk = lambda shape: torch.rand(shape, generator=gen).to(dtype)
+    else:
+        mk = lambda shape: torch.randn(shape, generator=gen).to(dtype)
+    full = [a + b for a, b in zip(q_lens, hist)]
+    ks = [mk((max(l, 1), hkv, d))[:l] for l in full]
+    vs = [mk((max(l, 1), hkv, d))[:l] for l in full]
+    T = sum(q_lens)
+    q = mk((T + 3, hq, d))                                 # 3 rows owned by no sequence
+    kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=seed, dtype=dtype)
+    start = torch.tensor([sum(q_lens[:i]) for i in range(len(q_lens))])
+    ql, kl = torch.tensor(q_lens), torch.tensor(full)
+    ref = oa.paged_prefill(q, kc, vc, table, start, ql, kl, sm_scale=sm_scale, window=window,
+                           softcap=softcap)
+    o = torch.full((T + 3, hq, d), 9.0, dtype=dtype, device=dev)
+    ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(dev), start.to(dev),
+                              ql.to(dev), kl.to(dev), max_seqlen or max(q_lens),
+                              window_size=window, sm_scale=sm_scale, logit_softcapping=softcap)
+    assert ret is None
+    out = o.cpu()
+    assert (out[T:] == 9.0).all()                         # rows outside every sequence untouched
+    assert torch.isfinite(out.float()).all()              # NaN-filled unused cache never read
+    torch.testing.assert_close(out[:T].float(), ref[:T].float(), rtol=tol, atol=tol)
+    return out[:T], ref[:T]
+
+
+# the reference's own prefill case (test_paged_attention.py:244-255): seq_lens [30,50,70,90]
+# after histories [50,40,30,20], heads (8,2)/(2,2), page 16, fp16, uniform inputs; head dims
+# moved to the supported 64/128
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (2, 2)])
+@pytest.mark.parametrize("d", [64, 128])
+def test_reference_prefill_cases(dev, hq, hkv, d):
+    out, ref = _run_case(dev, [30, 50, 70, 90], [50, 40, 30, 20], hq, hkv, d, 16, torch.float16,
+                         uniform=True)
+    torch.testing.assert_close(out.float(), ref.float(), rtol=1e-5, atol=1e-3)
+
+
+# the reference's window case (test_paged_attention.py:291-303): window 32 on the same lengths
+@pytest.mark.parametrize("d", [64, 128])
+def test_reference_window_case(dev, d):
+    out, ref = _run_case(dev, [30, 50, 70, 90], [50, 40, 30, 20], 4, 2, d, 16, torch.float16,
+                         uniform=True, window=32)
+    torch.testing.assert_close(out.float(), ref.float(), rtol=1e-5, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("page", [16, 64, 48])
+def test_length_edges(dev, dtype, page):
+    # query / history lengths around the 64-key tile, the 128-row block and the page size
+    q_lens = [1, 2, 63, 64, 65, 127, 128, 129, 200, 257, 5, 0]
+    hist = [0, 63, 1, 64, 127, 0, 128, 300, 77, 1, 1000, 10]
+    _run_case(dev, q_lens, hist, 8, 2, 128, page, dtype)
+
+
+def test_no_history_equals_varlen_prefill(dev):
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    q_lens = [100, 333, 64]
+    out, _ = _run_case(dev, q_lens, [0, 0, 0], 8, 2, 128, 64, torch.bfloat16, seed=3)
+    gen = torch.Generator().manual_seed(126)
+    mk = lambda shape: torch.randn(shape, generator=gen).to(torch.bfloat16)
+    ks = [mk((l, 2, 128)) for l in q_lens]
+    vs = [mk((l, 2, 128)) for l in q_lens]
+    q = mk((sum(q_lens) + 3, 8, 128))[:sum(q_lens)]
+    o = torch.empty_like(q, device=dev)
+    start = torch.tensor([0, 100, 433], dtype=torch.int32, device=dev)
+    context_attention_fwd(q.to(dev), torch.cat(ks).to(dev), torch.cat(vs).to(dev), o, start,
+                          torch.tensor(q_lens, dtype=torch.int32, device=dev), max(q_lens))
+    assert torch.equal(o.cpu(), out)                      # same kernel body, same tile order
+
+
+@pytest.mark.parametrize("window", [1, 31, 64, 200, 5000])
+def test_sliding_window(dev, window):
+    _run_case(dev, [1, 70, 130, 300], [500, 40, 0, 129], 8, 2, 128, 16, torch.bfloat16, window=window)
+
+
+@pytest.mark.parametrize("softcap", [0.5, 30.0])
+def test_logit_softcapping(dev, softcap):
+    _run_case(dev, [70, 130, 9], [40, 0, 300], 4, 4, 64, 32, torch.float16, softcap=softcap)
+
+
+def test_window_and_softcap_and_scale(dev):
+    _run_case(dev, [70, 130, 9], [40, 0, 300], 8, 1, 128, 16, torch.bfloat16, softcap=20.0, window=50,
+              sm_scale=0.2)
+
+
+def test_large_chunked_prefill(dev):
+    # one 128-row block far into a long context, the chunked-prefill shape
+    _run_case(dev, [512, 256], [3000, 1500], 8, 2, 128, 64, torch.bfloat16, seed=5)
+
+
+def test_grid_larger_than_needed_and_rejects(dev):
+    from dlcompiler_amd import _lib
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+
+    _run_case(dev, [10, 20], [5, 0], 2, 2, 64, 16, torch.float16, max_seqlen=1000)
+    q = torch.zeros(8, 2, 96, dtype=torch.float16, device=dev)          # unsupported head dim
+    kc = torch.zeros(4, 16, 2, 96, dtype=torch.float16, device=dev)
+    with pytest.raises(_lib.DlblasHipError):
+        paged_attention_fwd(q, kc, kc, torch.empty_like(q), torch.zeros(2, 2, dtype=torch.int32, device=dev),
+                            torch.tensor([0, 4], device=dev), torch.tensor([4, 4], device=dev),
+                            torch.tensor([4, 4], device=dev), 4)

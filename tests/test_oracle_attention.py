@@ -101,3 +101,53 @@ def test_window_and_softcap_closed_forms():
                                rtol=1e-2, atol=1e-2)
     flat = oa.paged_decode(q, kc, vc, table, n, softcap=1e-4)
     torch.testing.assert_close(flat[0, 0].float(), vs[0][:, 0].float().mean(0), rtol=2e-2, atol=2e-2)
+
+
+def _paged_prefill_case(q_lens, hist, hq=4, hkv=2, d=16, page=16, seed=0):
+    full = [a + b for a, b in zip(q_lens, hist)]
+    ks = [_rand((l, hkv, d), 10 + i) for i, l in enumerate(full)]
+    vs = [_rand((l, hkv, d), 20 + i) for i, l in enumerate(full)]
+    q = _rand((sum(q_lens), hq, d), 3)
+    kc, vc, table = oa.make_paged_cache(ks, vs, page=page, seed=seed)
+    start = torch.tensor([sum(q_lens[:i]) for i in range(len(q_lens))])
+    return q, ks, vs, kc, vc, table, start, torch.tensor(q_lens), torch.tensor(full)
+
+
+def test_paged_prefill_reduces_to_prefill_and_decode():
+    q_lens, hist = [30, 50, 7, 1], [50, 0, 30, 20]
+    q, ks, vs, kc, vc, table, start, ql, kl = _paged_prefill_case(q_lens, hist)
+    out = oa.paged_prefill(q, kc, vc, table, start, ql, kl)
+    # no history: packed varlen prefill of the same tokens
+    ref1 = oa.prefill_attention(q[30:80], ks[1], vs[1], torch.tensor([0]), torch.tensor([50]))
+    assert torch.equal(out[30:80], ref1)
+    # every query row alone is a decode step over the context that ends at its position
+    for b in range(4):
+        for i in (0, q_lens[b] - 1):
+            ctx = hist[b] + i + 1
+            row = oa.paged_decode(q[start[b] + i][None], kc, vc, table[b][None], torch.tensor([ctx]))
+            assert torch.equal(out[start[b] + i], row[0])
+    # additive-bias formulation of the reference test (key j hidden when j - i > history)
+    b = 0
+    kk = ks[b].float().repeat_interleave(2, dim=1).permute(1, 2, 0)            # [Hq, D, Lk]
+    vv = vs[b].float().repeat_interleave(2, dim=1).transpose(0, 1)             # [Hq, Lk, D]
+    qq = q[:30].float().transpose(0, 1)                                        # [Hq, Lq, D]
+    i = torch.arange(30)[:, None]
+    j = torch.arange(80)[None, :]
+    bias = ((j - i) > hist[b]).float() * -1e30
+    p = torch.softmax(qq @ kk / math.sqrt(16) + bias, dim=-1).to(q.dtype).float()
+    torch.testing.assert_close(out[:30].float(), (p @ vv).transpose(0, 1), rtol=2e-2, atol=2e-2)
+
+
+def test_paged_prefill_window():
+    q_lens, hist = [30, 12], [50, 40]
+    q, ks, vs, kc, vc, table, start, ql, kl = _paged_prefill_case(q_lens, hist)
+    base = oa.paged_prefill(q, kc, vc, table, start, ql, kl)
+    assert torch.equal(oa.paged_prefill(q, kc, vc, table, start, ql, kl, window=1000), base)
+    out = oa.paged_prefill(q, kc, vc, table, start, ql, kl, window=8)
+    # each row: decode over the context ending at its position with the same window
+    for b in range(2):
+        for i in range(q_lens[b]):
+            ctx = hist[b] + i + 1
+            row = oa.paged_decode(q[start[b] + i][None], kc, vc, table[b][None], torch.tensor([ctx]),
+                                  window=8)
+            assert torch.equal(out[start[b] + i], row[0])
