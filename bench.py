@@ -396,6 +396,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first launch an elementwise copy of 1 GiB (fp32 x * 1 -> y) three times: "
+                         "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the operators are single-device; "
@@ -409,6 +412,14 @@ def main():
     _lib.load()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        x = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        y = torch.empty_like(x)
+        for _ in range(3):
+            torch.mul(x, 1.0, out=y)
+        torch.cuda.synchronize()
+        del x, y
+        torch.cuda.empty_cache()
     names = list(WORKLOADS) if args.workload == "all" else [args.workload]
     primary = PRIMARY if args.workload == "all" else args.workload
     results = {}
