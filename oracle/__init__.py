@@ -17,7 +17,14 @@ Pinning status (what, other than the formula itself, each function is checked ag
                                     Python loop and to its invariants
 * ``attention.prefill_attention``   pinned: torch scaled_dot_product_attention, closed forms
 * ``attention.paged_decode``        pinned: same dense routine after an independent gather,
-                                    page-permutation invariance
+                                    page-permutation invariance; window = shorter context,
+                                    soft-cap limits (identity / mean of V)
+* ``attention.paged_prefill``       pinned: no history = prefill_attention, every row = a
+                                    paged_decode over the context ending there, the reference
+                                    test's additive-bias formulation
+* ``decoder_ops.fill_kv_cache``     pinned: page-by-page copy loop of the reference test
+* ``decoder_ops.rms_norm``          pinned: torch.nn.functional.rms_norm, fp64 evaluation
+* ``decoder_ops.apply_rotary_pos_emb``  pinned: complex rotation identity, norm preservation
 * ``fp8.per_token_group_quant`` / ``fp8.fused_moe_fp8``  parity unpinned w.r.t. the reference
                                     (no fp8 MoE exists there); pinned to torch's own e4m3fn
                                     cast, round-trip bounds and an fp64 dense evaluation
