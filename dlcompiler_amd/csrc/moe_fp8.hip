@@ -137,8 +137,11 @@ __device__ __forceinline__ f32x4 mfma_16bit(const i32x8& a, const i32x8& b, f32x
 //                epilogue silu(gate) * up -> fp8 + per-128 scale, rows kept in sorted order.
 // GATED = false: down GEMM, tile = 256 cols, epilogue * routing weight -> out[slot, n].
 // BM = rows (routing slots) per workgroup = the alignment block of the routing (64 or 128).
+#ifndef DLB_MOE_OCC
+#define DLB_MOE_OCC 2
+#endif
 template <bool GATED, int DT, int BM, int QT>
-__global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
+__global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
   constexpr int kBM = BM;
   constexpr int MT = BM / 16;          // 16-token sub-tiles
   constexpr int SKC = 2;               // 128-byte K chunks per activation stage
@@ -176,21 +179,27 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
 
   if (tid < kBM) sid_lds[tid] = p.sorted_ids[row0 + tid];
   static_assert(BM == 64 || BM == 128, "BM");
+  static_assert(AU == SKC * (BM / 32), "staging units per thread");
 
-  // ---- activation chunk staging: thread -> (row = tid / 4, 32-byte segment = tid % 4)
+  // ---- activation chunk staging.  Data: 8 consecutive lanes fetch one row's 128-byte chunk
+  // (a full cache line per row and instruction), 32 rows per pass, BM / 32 passes per chunk.
+  // Scales: thread (row = tid / TPR, chunk = tid % TPR < SKC) fetches one float per stage.
+  constexpr int RP = BM / 32;            // row passes per chunk
   const int arow = tid / TPR, aseg = tid % TPR;
-  const unsigned char* a_ptr;
+  const int prow = tid >> 3, piece = tid & 7;
+  const unsigned char* a_ptr[RP];
   const float* as_ptr;
   {
-    int64_t src_row;
-    if (GATED) {
-      const int sid = p.sorted_ids[row0 + arow];
-      src_row = min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
-    } else {
-      src_row = row0 + arow;
-    }
-    a_ptr = p.a + src_row * K;
-    as_ptr = QT == 0 ? p.a_scale + src_row * KC : nullptr;
+    auto src_row_of = [&](int r) -> int64_t {
+      if (GATED) {
+        const int sid = p.sorted_ids[row0 + r];
+        return min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
+      }
+      return row0 + r;
+    };
+#pragma unroll
+    for (int k = 0; k < RP; ++k) a_ptr[k] = p.a + src_row_of(32 * k + prow) * K + 16 * piece;
+    as_ptr = QT == 0 ? p.a_scale + src_row_of(arow) * KC : nullptr;
   }
 
   // ---- weight fragments: sub-tile j of this wave covers 16 output columns
@@ -252,16 +261,15 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
     const int kc0 = st * SKC;
 #pragma unroll
     for (int u = 0; u < AU; ++u) {
-      const int byte = aseg * (16 * AU) + 16 * u;  // inside the stage's SKC * 128 bytes
-      const int kc = min(kc0 + (byte >> 7), KC - 1);
-      areg[u] = *(const u32x4*)(a_ptr + kc * 128 + (byte & 127));
+      const int kc = min(kc0 + u / RP, KC - 1);
+      areg[u] = *(const u32x4*)(a_ptr[u % RP] + kc * 128);
     }
     if (QT == 0 && aseg < SKC) asreg = as_ptr[min(kc0 + aseg, KC - 1)];
   };
   auto store_a = [&](int buf) {
-    unsigned char* dst = a_lds[buf] + arow * kARow + aseg * (16 * AU);
+    unsigned char* dst = a_lds[buf] + prow * kARow + 16 * piece;
 #pragma unroll
-    for (int u = 0; u < AU; ++u) *(u32x4*)(dst + 16 * u) = areg[u];
+    for (int u = 0; u < AU; ++u) *(u32x4*)(dst + (u % RP) * 32 * kARow + (u / RP) * 128) = areg[u];
     if (QT == 0 && aseg < SKC) as_lds[buf][aseg][arow] = asreg;
   };
   auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
@@ -330,6 +338,9 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
               pc[j] = mfma_fp8(breg[slot][j], xq[t & 1]);
               acc[pm][j] += pp[j] * psc[j];
             }
+            // keep the retiring FMAs next to these MFMAs (the optimiser would otherwise sink
+            // them into one long VALU run with nothing to overlap)
+            asm volatile("" : "+v"(acc[pm][0]), "+v"(acc[pm][1]), "+v"(acc[pm][2]), "+v"(acc[pm][3]));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               pp[j] = pc[j];
@@ -400,7 +411,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
         for (int i = 0; i < 4; ++i) {
           const float gate = acc[mt][jg][i];
           const float up = acc[mt][jg + 2][i];
-          const float v = gate / (1.0f + __expf(-gate)) * up;
+          const float v = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;  // 1-ulp reciprocal
           h[mt][jg][i] = v;
           amax[mt] = fmaxf(amax[mt], fabsf(v));
         }
@@ -416,11 +427,12 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
       const int r = 16 * mt + c;
       const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
       const float scale = fmaxf(m, kQuantEps) / kFp8Max;
+      const float inv = __builtin_amdgcn_rcpf(scale);  // the stored scale stays exact
       const int64_t orow = row0 + r;
 #pragma unroll
       for (int jg = 0; jg < 2; ++jg) {
-        const unsigned int q = pack4_fp8(h[mt][jg][0] / scale, h[mt][jg][1] / scale,
-                                         h[mt][jg][2] / scale, h[mt][jg][3] / scale);
+        const unsigned int q = pack4_fp8(h[mt][jg][0] * inv, h[mt][jg][1] * inv,
+                                         h[mt][jg][2] * inv, h[mt][jg][3] * inv);
         *(unsigned int*)(p.hq + orow * p.I + nt * 128 + wave * 32 + 16 * jg + 4 * g) = q;
       }
       if (wave == 0 && g == 0) p.hs[orow * (p.I >> 7) + scol] = scale;
@@ -444,6 +456,400 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_fp8_kernel(const MoeGemmParam
           }
         }
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Wide grouped GEMM: 128 routing slots x 256 output columns per workgroup of 8 waves (one
+// workgroup per CU).  Twice the rows per weight byte of the 64-row kernel, which is what the
+// L2 -> CU path rewards.  Both operands go HBM/L2 -> LDS with direct-to-LDS loads (no staging
+// registers, no ds_write): per 128-byte K chunk 256 weight rows + 128 activation rows, each
+// row 128 bytes with its eight 16-byte pieces XOR-swizzled by (row >> 1) & 7 so that the
+// ds_read_b128 of an MFMA fragment (16 rows x 2 pieces per lane) runs at full LDS rate.
+// Rings: weights 3 slots (issued two chunks ahead of use), activations 3 slots (one chunk
+// ahead).  Wave (rg, cg) owns rows 64*rg.. and 64 columns; per chunk it reads its 4 weight
+// fragments once (double-buffered in registers, fetched half a chunk early) and one
+// activation fragment per 16-row step.  One barrier per chunk, placed in the middle of the
+// chunk's MFMAs so nobody waits for LDS right after it.
+// Weights may be row-major (8 lanes fetch one row's 128-byte line) or operand-order.
+// ---------------------------------------------------------------------------------------
+template <bool GATED, int DT, int QT>
+__global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmParams p) {
+  constexpr int BM = 128, BN = 256, MT = 4;
+  constexpr int kWSlot = BN * 128;  // bytes of one weight ring slot
+  constexpr int kXSlot = BM * 128;  // bytes of one activation ring slot
+  constexpr int kSC = 16;           // chunks of activation scales resident in LDS
+  __shared__ __attribute__((aligned(1024))) unsigned char w_lds[3 * kWSlot];
+  __shared__ __attribute__((aligned(1024))) unsigned char x_lds[3 * kXSlot];
+  __shared__ float as_lds[kSC][BM];
+  __shared__ float ws_lds[2][kSC];  // block scales of the tile's two 128-column weight blocks
+  __shared__ float red_lds[4][BM];
+  __shared__ int32_t sid_lds[BM];
+
+  const int per_xcd = gridDim.x >> 3;
+  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= p.grid_real) return;
+  const int mb = logical % p.num_mblocks;
+  const int nt = logical / p.num_mblocks;
+  const int e_global = p.expert_ids[mb];
+  const int e = e_global - p.expert_offset;
+  if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
+
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave id, kept in scalar registers
+  const int lane = tid & 63;
+  const int g = lane >> 4;
+  const int c = lane & 15;
+  const int rg = w >> 2;  // waves w and w + 4 share a SIMD: give them different row groups
+  const int cg = w & 3;
+  const int row0 = mb * BM;
+  const int K = p.K, KC = p.KC;
+
+  if (tid < BM) sid_lds[tid] = p.sorted_ids[row0 + tid];
+
+  auto src_row_of = [&](int r) -> int {
+    if (GATED) {
+      const int sid = p.sorted_ids[row0 + r];
+      return min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
+    }
+    return row0 + r;
+  };
+
+  // ---- direct-to-LDS staging: instruction = 8 rows x 128 bytes, lane -> (row, physical piece)
+  const int drow = lane >> 3, dpc = lane & 7;
+  uint32_t w_voff[4], x_voff[2];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = 32 * w + 8 * q + drow;  // tile-local weight row
+    int n;
+    if (GATED) n = (r < 128) ? nt * 128 + r : p.I + nt * 128 + (r - 128);
+    else n = nt * 256 + r;
+    n = min(n, p.N - 1);
+    const int lc = dpc ^ ((r >> 1) & 7);  // logical piece that lands in physical piece dpc
+    if (p.w_layout)
+      w_voff[q] = (uint32_t)(n >> 4) * (uint32_t)KC * 2048u + (uint32_t)(lc >> 2) * 1024u +
+                  (uint32_t)(((lc & 3) * 16 + (n & 15)) * 16);
+    else
+      w_voff[q] = (uint32_t)n * (uint32_t)K + (uint32_t)lc * 16u;
+  }
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int r = 16 * w + 8 * q + drow;
+    const int lc = dpc ^ ((r >> 1) & 7);
+    x_voff[q] = (uint32_t)src_row_of(r) * (uint32_t)K + (uint32_t)lc * 16u;
+  }
+  const unsigned char* wbase = p.w + (int64_t)e * p.N * K;
+  const int w_kc_stride = p.w_layout ? 2048 : 128;
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  // address = uniform base (scalar registers) + 32-bit lane offset: no 64-bit vector math
+  auto issue_w = [&](int kc, int slot) {
+    const uint32_t koff = (uint32_t)kc * (uint32_t)w_kc_stride;
+    unsigned char* dst = w_lds + slot * kWSlot + w * 4096;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_global_load_lds((gptr_t)(wbase + (uint32_t)(w_voff[q] + koff)),
+                                       (lptr_t)(dst + q * 1024), 16, 0, 0);
+  };
+  auto issue_x = [&](int kc, int slot) {
+    const uint32_t koff = (uint32_t)kc * 128u;
+    unsigned char* dst = x_lds + slot * kXSlot + w * 2048;
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      __builtin_amdgcn_global_load_lds((gptr_t)(p.a + (uint32_t)(x_voff[q] + koff)),
+                                       (lptr_t)(dst + q * 1024), 16, 0, 0);
+  };
+  // activation scales of chunks [kc0, kc0 + kSC) -> LDS (plain loads; 4 per thread)
+  auto load_scales = [&](int kc0) {
+    if (QT != 0) return;
+    const int r = tid & (BM - 1), kq = tid >> 7;
+    const float* sp = p.a_scale + (int64_t)src_row_of(r) * KC;
+#pragma unroll
+    for (int i = 0; i < kSC / 4; ++i) {
+      const int kk = kq * (kSC / 4) + i;
+      as_lds[kk][r] = sp[min(kc0 + kk, KC - 1)];
+    }
+    if (tid < 2 * kSC) {
+      const int which = tid / kSC, kk = tid % kSC;
+      const int blk = GATED ? (which ? (p.I >> 7) + nt : nt) : min(2 * nt + which, (p.N >> 7) - 1);
+      ws_lds[which][kk] = p.w_scale[((int64_t)e * (p.N >> 7) + blk) * KC + min(kc0 + kk, KC - 1)];
+    }
+  };
+
+  // ---- fragment reads: lane (c, g) takes pieces g and g + 4 of row (tile row + c)
+  // Per lane one base pointer per operand and half; slot and tile offsets are a scalar add and
+  // an immediate.  Column sub-tile j starts at tile-local weight row
+  //   gated: (j >> 1) * 128 + cg * 32 + (j & 1) * 16,   down: cg * 64 + j * 16.
+  const int lo_off = c * 128 + (((g) ^ (c >> 1)) & 7) * 16;
+  const int hi_off = c * 128 + (((g + 4) ^ (c >> 1)) & 7) * 16;
+  const int wcg = (GATED ? cg * 32 : cg * 64) * 128;
+  const unsigned char* w_lo = w_lds + wcg + lo_off;
+  const unsigned char* w_hi = w_lds + wcg + hi_off;
+  const unsigned char* x_lo = x_lds + rg * (64 * 128) + lo_off;
+  const unsigned char* x_hi = x_lds + rg * (64 * 128) + hi_off;
+  const float* as_base = &as_lds[0][64 * rg + c];
+  auto read_w = [&](int slot, i32x8 (&b)[4]) {
+    const unsigned char* bl = w_lo + slot * kWSlot;
+    const unsigned char* bh = w_hi + slot * kWSlot;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      constexpr int kUp = 128 * 128;  // gated: up rows follow the 128 gate rows
+      const int off = GATED ? (j >> 1) * kUp + (j & 1) * 2048 : j * 2048;
+      const u32x4 lo = *(const u32x4*)(bl + off);
+      const u32x4 hi = *(const u32x4*)(bh + off);
+      b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+                   (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    }
+  };
+  auto read_x = [&](int slot, int kc, int mt, i32x8& x, float& as) {
+    const u32x4 lo = *(const u32x4*)(x_lo + slot * kXSlot + mt * 2048);
+    const u32x4 hi = *(const u32x4*)(x_hi + slot * kXSlot + mt * 2048);
+    x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+              (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    as = QT == 0 ? as_base[(kc & (kSC - 1)) * BM + 16 * mt] : 1.0f;
+  };
+
+  // ---- weight block scales: wave-uniform, one per (128-column block, chunk), read from LDS
+  // (gated: block 0 = gate columns, 1 = up columns; down: the wave's own 128-column block)
+  const float* ws_row0 = ws_lds[GATED ? 0 : (cg >> 1)];
+  const float* ws_row1 = ws_lds[GATED ? 1 : (cg >> 1)];
+
+  f32x4 acc[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 pp[4];
+  float psc[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) pp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  i32x8 b0[4], b1[4];
+  i32x8 xq[2];
+  float asq[2];
+  float wsc[2] = {1.0f, 1.0f}, wsn[2] = {1.0f, 1.0f};
+
+  // prologue: scales, chunks 0..2 of the weights and 0..1 of the activations in flight
+  load_scales(0);
+  issue_x(0, 0);
+  issue_w(0, 0);
+  if (KC > 1) {
+    issue_x(1, 1);
+    issue_w(1, 1);
+  }
+  if (KC > 2) {
+    issue_w(2, 2);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | 10);  // vmcnt(10): chunk 0 landed, 10 newer loads may fly
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
+  }
+  __syncthreads();
+  read_w(0, b0);
+  read_x(0, 0, 0, xq[0], asq[0]);
+  if (QT == 0) {
+    wsc[0] = ws_row0[0];
+    wsc[1] = ws_row1[0];
+  }
+
+  // one 16-row step: 4 MFMAs, each followed by the FMAs retiring one product of the previous step
+  auto step = [&](const i32x8 (&b)[4], int mt, int cur) {
+    const int pm = (mt == 0) ? MT - 1 : mt - 1;
+    if constexpr (QT == 0) {
+      f32x4 pc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        pc[j] = mfma_fp8(b[j], xq[cur]);
+        acc[pm][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
+      }
+      // keep the retiring FMAs inside this step (they would otherwise be sunk past the
+      // following steps and run as one block with no MFMA to overlap)
+      asm volatile("" : "+v"(acc[pm][0]), "+v"(acc[pm][1]), "+v"(acc[pm][2]), "+v"(acc[pm][3]));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pp[j] = pc[j];
+      psc[0] = asq[cur] * wsc[0];
+      psc[1] = asq[cur] * wsc[1];
+    } else {
+      (void)pm;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[mt][j] = mfma_16bit<DT>(b[j], xq[cur], acc[mt][j]);
+    }
+  };
+  // ring positions as scalars rotated once per chunk (no modulo in the loop): slot of chunk
+  // kc (x_cur / w_cur), kc + 1 (x_nxt / w_nxt) and the one to refill (x_tgt: chunk kc + 2;
+  // the weights of chunk kc + 3 go where chunk kc was)
+  int x_cur = 0, x_nxt = 1, x_tgt = 2;
+  int w_cur = 0, w_nxt = 1, w_aft = 2;
+  auto rotate = [&]() {
+    wsc[0] = wsn[0];
+    wsc[1] = wsn[1];
+    const int xr = x_cur;
+    x_cur = x_nxt;
+    x_nxt = x_tgt;
+    x_tgt = xr;
+    const int wr = w_cur;
+    w_cur = w_nxt;
+    w_nxt = w_aft;
+    w_aft = wr;
+  };
+  auto do_chunk = [&](const i32x8 (&bc)[4], i32x8 (&bn)[4], int kc) {
+    const bool more = kc + 1 < KC;
+    read_x(x_cur, kc, 1, xq[1], asq[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    step(bc, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    read_x(x_cur, kc, 2, xq[0], asq[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    step(bc, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) {
+      // chunk kc + 1 has landed once every wave's own loads of it are back
+      if (kc + 2 < KC) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);  // W(kc + 2) may still fly
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      if (QT == 0 && ((kc + 1) & (kSC - 1)) == 0) {
+        // rare (K > 2048 bytes): next tile of activation scales; every wave is past its reads
+        // of the old tile once it has the step-3 fragment, so fetch that first
+        read_x(x_cur, kc, 3, xq[1], asq[1]);
+        __syncthreads();
+        load_scales(kc + 1);
+        __syncthreads();
+      } else {
+        __syncthreads();
+        read_x(x_cur, kc, 3, xq[1], asq[1]);
+      }
+      if (kc + 2 < KC) issue_x(kc + 2, x_tgt);
+      if (kc + 3 < KC) issue_w(kc + 3, w_cur);
+      read_w(w_nxt, bn);
+      if (QT == 0) {
+        wsn[0] = ws_row0[(kc + 1) & (kSC - 1)];
+        wsn[1] = ws_row1[(kc + 1) & (kSC - 1)];
+      }
+    } else {
+      read_x(x_cur, kc, 3, xq[1], asq[1]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    step(bc, 2, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) read_x(x_nxt, kc + 1, 0, xq[0], asq[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    step(bc, 3, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    rotate();
+  };
+  for (int kc = 0; kc < KC; kc += 2) {
+    do_chunk(b0, b1, kc);
+    if (kc + 1 < KC) do_chunk(b1, b0, kc + 1);
+  }
+  if constexpr (QT == 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
+  }
+
+  // ---- epilogues: lane holds slot row (64*rg + 16*mt + c), columns (sub-tile j) + 4*g + i.
+  // The output tile is assembled in LDS (the weight ring is free once every wave has left the
+  // main loop) and written out as whole rows: 16-byte pieces, a row's pieces on adjacent lanes.
+  const int rbase = 64 * rg;
+  unsigned char* stage = w_lds;
+  // copy `rows` x `row_bytes` from the staging tile to global rows given by dst_of(r) (nullptr: skip)
+  auto flush_rows = [&](int row_bytes, auto dst_of) {
+    const int ppr = row_bytes >> 4;            // 16-byte pieces per row
+    const int total = BM * ppr;
+    for (int u = tid; u < total; u += 512) {
+      const int r = u / ppr, pc = u - r * ppr;
+      unsigned char* dst = dst_of(r);
+      if (dst) *(u32x4*)(dst + 16 * pc) = *(const u32x4*)(stage + r * row_bytes + 16 * pc);
+    }
+  };
+  if (GATED && QT == 1) {
+    // rounding points of the reference pipeline (fused_moe.py:166,351-352)
+    __syncthreads();  // all waves are done with the rings
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      unsigned short* dst = (unsigned short*)stage + (rbase + 16 * mt + c) * 128 + cg * 32 + 4 * g;
+#pragma unroll
+      for (int jg = 0; jg < 2; ++jg) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const unsigned int gu = Elem<DT>::pack(acc[mt][jg][i], acc[mt][jg + 2][i]);
+          const float gate = Elem<DT>::lo(gu), up = Elem<DT>::hi(gu);
+          const float sg = Elem<DT>::lo(Elem<DT>::pack(gate / (1.0f + __expf(-gate)), 0.0f));
+          v[i] = sg * up;
+        }
+        u32x2 o2;
+        o2[0] = Elem<DT>::pack(v[0], v[1]);
+        o2[1] = Elem<DT>::pack(v[2], v[3]);
+        *(u32x2*)(dst + 16 * jg) = o2;
+      }
+    }
+    __syncthreads();
+    flush_rows(256, [&](int r) -> unsigned char* {
+      return p.hq + ((int64_t)(row0 + r) * p.I + nt * 128) * 2;
+    });
+  } else if (GATED) {
+    float h[MT][2][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float amax = 0.0f;
+#pragma unroll
+      for (int jg = 0; jg < 2; ++jg) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float gate = acc[mt][jg][i];
+          const float up = acc[mt][jg + 2][i];
+          const float v = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;  // 1-ulp reciprocal
+          h[mt][jg][i] = v;
+          amax = fmaxf(amax, fabsf(v));
+        }
+      }
+      amax = fmaxf(amax, __shfl_xor(amax, 16));
+      amax = fmaxf(amax, __shfl_xor(amax, 32));
+      if (g == 0) red_lds[cg][rbase + 16 * mt + c] = amax;
+    }
+    __syncthreads();  // row maxima visible; all waves are done with the rings
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int r = rbase + 16 * mt + c;
+      const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
+      const float scale = fmaxf(m, kQuantEps) / kFp8Max;
+      const float inv = __builtin_amdgcn_rcpf(scale);  // the stored scale stays exact
+#pragma unroll
+      for (int jg = 0; jg < 2; ++jg) {
+        const unsigned int q = pack4_fp8(h[mt][jg][0] * inv, h[mt][jg][1] * inv,
+                                         h[mt][jg][2] * inv, h[mt][jg][3] * inv);
+        *(unsigned int*)(stage + r * 128 + cg * 32 + 16 * jg + 4 * g) = q;
+      }
+      if (cg == 0 && g == 0) p.hs[(int64_t)(row0 + r) * (p.I >> 7) + nt] = scale;
+    }
+    __syncthreads();
+    flush_rows(128, [&](int r) -> unsigned char* {
+      return p.hq + (int64_t)(row0 + r) * p.I + nt * 128;
+    });
+  } else {
+    __syncthreads();  // all waves are done with the rings (and sid_lds is long visible)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int r = rbase + 16 * mt + c;
+      const int sid = sid_lds[r];
+      const float rw = sid < p.numel ? p.topk_w[sid] : 0.0f;
+      unsigned short* dst = (unsigned short*)stage + r * 256 + cg * 64 + 4 * g;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u32x2 o2;
+        o2[0] = Elem<DT>::pack(acc[mt][j][0] * rw, acc[mt][j][1] * rw);
+        o2[1] = Elem<DT>::pack(acc[mt][j][2] * rw, acc[mt][j][3] * rw);
+        *(u32x2*)(dst + 16 * j) = o2;
+      }
+    }
+    __syncthreads();
+    const int ncols = min(256, p.N - nt * 256);  // multiple of 128
+    const int ppr = ncols >> 3;                  // 16-byte pieces of a row that exist
+    for (int u = tid; u < BM * 32; u += 512) {
+      const int r = u >> 5, pc = u & 31;
+      const int sid = sid_lds[r];
+      if (sid < p.numel && pc < ppr)
+        *(u32x4*)((unsigned short*)p.out + (int64_t)sid * p.N + nt * 256 + 8 * pc) =
+            *(const u32x4*)(stage + r * 512 + 16 * pc);
     }
   }
 }
@@ -511,18 +917,27 @@ namespace {
 template <bool GATED, int QT>
 int launch_moe_gemm(const MoeGemmParams& p, int dtype, int block_m, hipStream_t s) {
   const uint32_t grid = (uint32_t)(ceil_div(p.grid_real, 8) * 8);
-#define DLB_LAUNCH_GEMM(DT_, BM_) \
-  hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, BM_, QT>), dim3(grid), dim3(256), 0, s, p)
+  // the 128-row kernel stores whole 16-byte pieces and addresses activation rows with 32 bits
+  if (block_m == 128) {
+    if ((p.hq && !aligned16(p.hq)) || (p.out && !aligned16(p.out))) return DLB_ERR_UNSUPPORTED;
+    const int64_t a_rows = GATED ? p.num_tokens : (int64_t)p.num_mblocks * 128;
+    if (a_rows * p.K >= (int64_t)0xffffffffu) return DLB_ERR_UNSUPPORTED;
+  }
+#define DLB_LAUNCH_GEMM(DT_) \
+  hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, 64, QT>), dim3(grid), dim3(256), 0, s, p)
+#define DLB_LAUNCH_WIDE(DT_) \
+  hipLaunchKernelGGL((moe_gemm_wide_kernel<GATED, DT_, QT>), dim3(grid), dim3(512), 0, s, p)
   if (dtype == DLB_DTYPE_BF16) {
-    if (block_m == 128) DLB_LAUNCH_GEMM(DLB_DTYPE_BF16, 128);
-    else DLB_LAUNCH_GEMM(DLB_DTYPE_BF16, 64);
+    if (block_m == 128) DLB_LAUNCH_WIDE(DLB_DTYPE_BF16);
+    else DLB_LAUNCH_GEMM(DLB_DTYPE_BF16);
   } else if (dtype == DLB_DTYPE_F16) {
-    if (block_m == 128) DLB_LAUNCH_GEMM(DLB_DTYPE_F16, 128);
-    else DLB_LAUNCH_GEMM(DLB_DTYPE_F16, 64);
+    if (block_m == 128) DLB_LAUNCH_WIDE(DLB_DTYPE_F16);
+    else DLB_LAUNCH_GEMM(DLB_DTYPE_F16);
   } else {
     return DLB_ERR_UNSUPPORTED;
   }
 #undef DLB_LAUNCH_GEMM
+#undef DLB_LAUNCH_WIDE
   return launch_status();
 }
 
