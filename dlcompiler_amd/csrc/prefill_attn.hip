@@ -83,7 +83,7 @@ template <int D>
 struct Smem {
   static constexpr int kRowBytes = D * 2;           // K: [64][D], 16-byte chunks XOR-swizzled
   static constexpr int kBytes = kTileN * kRowBytes;
-  static constexpr int vRowBytes = kTileN * 2 + 16;  // V^T: [D][64] + pad
+  static constexpr int vRowBytes = kTileN * 2;       // V^T: [D][64], 16-byte units XOR-swizzled
   static constexpr int vBytes = D * vRowBytes;
   static constexpr int stage = kBytes + vBytes;
 };
@@ -224,7 +224,9 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
         const unsigned int hi01 = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], 0x07060302u);
         const unsigned int hi23 = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], 0x07060302u);
         const int d0 = 8 * st_dg + 2 * w;
-        const int sw = (d0 >> 4) & 7;  // same for d0 and d0 + 1; spreads the 16 dim groups
+        // unit swizzle (same for d0 and d0 + 1): with it the fragment reads below run at the
+        // full LDS rate and these transposing writes at half of theirs
+        const int sw = ((d0 >> 1) ^ (d0 >> 4)) & 7;
         unsigned char* row = vs + d0 * SM::vRowBytes + ((st_unit ^ sw) << 4) + (st_half << 3);
         *(u32x2*)(row) = u32x2{lo01, lo23};
         *(u32x2*)(row + SM::vRowBytes) = u32x2{hi01, hi23};
@@ -256,18 +258,33 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     const unsigned char* vs = ks + SM::kBytes;
 
     // ---- S^T = K . Q^T : two 32-key tiles x 32 queries (raw scores)
+    // k-step outer, key tile inner: two independent accumulator chains, and the K fragments
+    // are fetched from LDS two k-steps ahead of the MFMAs that consume them
     f32x16 s[2];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
-      const int krow_i = 32 * nt + col;
-      const unsigned char* krow = ks + krow_i * SM::kRowBytes;
-      const int ksw = krow_i & (DG - 1);
+    {
+      const unsigned char* krow0 = ks + col * SM::kRowBytes;
+      const unsigned char* krow1 = ks + (32 + col) * SM::kRowBytes;
+      const int ksw = col & (DG - 1);  // (32 + col) & (DG - 1) is the same
+      auto ldk = [&](int kstep, u32x4 (&a)[2]) {
+        const int off = ((2 * kstep + hh) ^ ksw) << 4;
+        a[0] = *(const u32x4*)(krow0 + off);
+        a[1] = *(const u32x4*)(krow1 + off);
+      };
+      constexpr int kAhead = 2;
+      u32x4 ka[kAhead + 1][2];
+#pragma unroll
+      for (int q = 0; q < kAhead; ++q) ldk(q, ka[q]);
 #pragma unroll
       for (int kstep = 0; kstep < KS; ++kstep) {
-        const u32x4 a = *(const u32x4*)(krow + (((2 * kstep + hh) ^ ksw) << 4));
-        s[nt] = Mma32<DT>::run(a, qf[kstep], s[nt]);
+        if (kstep + kAhead < KS) ldk(kstep + kAhead, ka[(kstep + kAhead) % (kAhead + 1)]);
+        __builtin_amdgcn_sched_barrier(0);  // keep the fetch ahead of the MFMAs (it would be sunk)
+        s[0] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][0], qf[kstep], s[0]);
+        s[1] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][1], qf[kstep], s[1]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
@@ -329,7 +346,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const int d = 32 * mt + col;
-          const int sw = (d >> 4) & 7;
+          const int sw = ((d >> 1) ^ (d >> 4)) & 7;
           const u32x4 a = *(const u32x4*)(vs + d * SM::vRowBytes + ((unit ^ sw) << 4));
           o[mt] = Mma32<DT>::run(a, pf, o[mt]);
         }
