@@ -85,14 +85,18 @@ constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
 // of the SAME (sequence, KV chunk), so the waves of a workgroup read neighbouring 256-byte
 // head slices of the same token rows at the same time (whole 2 KB token rows in flight).
 template <int DT, int D, int WPB, bool POW2>
-__global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(64 * WPB, 2) void paged_decode_split_kernel(const DecodeParams p) {
   constexpr int KS = D / 32;   // MFMA k-steps over the head dim
   constexpr int MT = D / 16;   // 16-row tiles of O^T
   constexpr int DG = D / 8;    // 8-dim groups per key row
 
-  const int split = blockIdx.x;
+  // grid: x = (kv head, head chunk) unit, y = KV chunk, z = sequence.  The unit is the fastest
+  // index, so workgroups that start together read the 256-byte head slices of the SAME token
+  // rows at the same time: whole 2 KB cache rows are in flight together and DRAM pages are hit
+  // while open.
+  const int split = blockIdx.y;
   const int wave = threadIdx.x >> 6;
-  const int unit = blockIdx.y * WPB + wave;
+  const int unit = blockIdx.x * WPB + wave;
   const int kvh = unit / p.hchunks;
   const int hchunk = unit - kvh * p.hchunks;
   const int b = blockIdx.z;
@@ -142,65 +146,69 @@ __global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const Deco
   constexpr int VPASS = 4 / VL;                  // passes per 16-key sub-tile
   const int dg = lane % DG, kgl = lane / DG;     // lanes with kgl >= VL idle (D < 128)
 
-  for (int t0 = k_begin; t0 < k_end; t0 += kTile) {
-    // ---- K tile: 4 sub-tiles of 16 keys, straight into A-operand registers ----
-    u32x4 kf[4][KS];
-    u32x4 vr[4][VPASS][4];
+  // The chunk is walked in half tiles of 32 keys (one k-step of the second product).  The loads
+  // of half tile h + 1 are issued before half tile h is computed, so every wave keeps 16 KB of
+  // requests in flight while it works; a wave's V^T staging buffer is private and LDS
+  // operations of one wave execute in order, so no barrier is needed.
+  struct HalfTile {
+    u32x4 kf[2][KS];          // K: 2 sub-tiles of 16 keys, already in A-operand layout
+    u32x4 vr[2][VPASS][4];    // V: per lane 4 consecutive keys x 8 dims per pass
+  };
+  auto load_half = [&](int h0, HalfTile& f) {
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
-      const int base_key = min(t0 + 16 * sub, ctx - 1);  // uniform; clamp: never read past ctx
+    for (int sub = 0; sub < 2; ++sub) {
+      const int base_key = min(h0 + 16 * sub, ctx - 1);  // uniform; clamp: never read past ctx
       const int pi = POW2 ? (base_key >> p.page_shift) : (base_key / p.page);
       const int64_t pg = (int64_t)bt[pi];
       const int page_key0 = pi * p.page;
       {
-        const int key = min(t0 + 16 * sub + c, ctx - 1);
+        const int key = min(h0 + 16 * sub + c, ctx - 1);
         const unsigned char* base = kbytes + pg * p.k_sp * 2;
         // K rows are read as two half-line (64-byte) pieces by consecutive k-steps: keep them
         // cacheable so the second piece hits the line the first one brought in
         const uint32_t off = (uint32_t)(key - page_key0) * k_tok_bytes + 16u * g;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kf[sub][ks] = *(const u32x4*)(base + off + 64 * ks);
+        for (int ks = 0; ks < KS; ++ks) f.kf[sub][ks] = *(const u32x4*)(base + off + 64 * ks);
       }
-      // ---- V: each lane takes 4 consecutive keys x 8 dims
       {
         const unsigned char* base = vbytes + pg * p.v_sp * 2;
 #pragma unroll
         for (int ps = 0; ps < VPASS; ++ps) {
-          const int key0 = min(t0 + 16 * sub + 4 * (ps * VL + kgl), ctx - 1);
+          const int key0 = min(h0 + 16 * sub + 4 * (ps * VL + kgl), ctx - 1);
           const int room = ctx - 1 - key0;
           if (kgl < VL) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const uint32_t off = (uint32_t)(key0 - page_key0 + min(r, room)) * v_tok_bytes + 16u * dg;
-              vr[sub][ps][r] = __builtin_nontemporal_load((const u32x4*)(base + off));
+              f.vr[sub][ps][r] = __builtin_nontemporal_load((const u32x4*)(base + off));
             }
           }
         }
       }
     }
-
+  };
+  // st = parity of the half tile inside its 64-key tile = which 4 units of a V^T row it uses
+  auto compute_half = [&](int h0, const HalfTile& f, int st) {
     // ---- S^T = K . Q^T (rows = keys, cols = query heads) ----
-    f32x4 s[4];
+    f32x4 s[2];
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
+    for (int sub = 0; sub < 2; ++sub) {
       s[sub] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) s[sub] = Mma16<DT>::run(kf[sub][ks], qf[ks], s[sub]);
+      for (int ks = 0; ks < KS; ++ks) s[sub] = Mma16<DT>::run(f.kf[sub][ks], qf[ks], s[sub]);
     }
 
-    // ---- V^T into LDS: Vt[d][pos], pos = 32*s + 8*g' + 4*a + r for key 32*s + 16*a + 4*g' + r
-    __syncthreads();  // previous tile's operand reads are done
+    // ---- V^T into LDS: Vt[d][pos], pos = 32*st + 8*g' + 4*a + r for key 32*st + 16*a + 4*g' + r
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
+    for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
       for (int ps = 0; ps < VPASS; ++ps) {
         if (kgl < VL) {
-          // key group kg = 4 * sub + (ps * VL + kgl) inside the 64-key tile
-          const int unit = 4 * (sub >> 1) + ps * VL + kgl;  // 16-byte unit inside the row
-          const int half = sub & 1;                         // 8-byte half inside the unit
+          const int unit = 4 * st + ps * VL + kgl;  // 16-byte unit inside the row
+          const int half = sub;                     // 8-byte half inside the unit
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
-            const u32x4* v4 = vr[sub][ps];
+            const u32x4* v4 = f.vr[sub][ps];
             const unsigned int lo01 = __builtin_amdgcn_perm(v4[1][w], v4[0][w], 0x05040100u);
             const unsigned int lo23 = __builtin_amdgcn_perm(v4[3][w], v4[2][w], 0x05040100u);
             const unsigned int hi01 = __builtin_amdgcn_perm(v4[1][w], v4[0][w], 0x07060302u);
@@ -215,13 +223,13 @@ __global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const Deco
       }
     }
 
-    // ---- online softmax over this tile (log2 domain) ----
+    // ---- online softmax over these 32 keys (log2 domain) ----
     float mloc = -__builtin_inff();
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
+    for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = t0 + 16 * sub + 4 * g + i;
+        const int key = h0 + 16 * sub + 4 * g + i;
         float x = s[sub][i] * p.scale_log2e;
         if (p.softcap > 0.0f)
           x = p.softcap * tanhf(s[sub][i] * p.sm_scale / p.softcap) * 1.4426950408889634f;
@@ -232,44 +240,58 @@ __global__ __launch_bounds__(64 * WPB) void paged_decode_split_kernel(const Deco
     }
     mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float m_new = fmaxf(m_run, mloc);  // finite: key t0 is always valid
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    const float m_new = fmaxf(m_run, mloc);
+    // a half tile can be entirely masked (sliding window, chunk tail): keep exponents finite
+    const float m_ref = (m_new == -__builtin_inff()) ? 0.0f : m_new;
+    if (__any(m_new > m_run)) {  // wave-uniform: skip the rescale when no maximum moved
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
+      l_run *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+    }
     m_run = m_new;
     float psum = 0.0f;
 #pragma unroll
-    for (int sub = 0; sub < 4; ++sub) {
+    for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float e = __builtin_amdgcn_exp2f(s[sub][i] - m_new);
+        const float e = __builtin_amdgcn_exp2f(s[sub][i] - m_ref);
         s[sub][i] = e;
         psum += e;
       }
     }
-    l_run = l_run * alpha + psum;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+    l_run += psum;
 
-    // P^T as B operand of step st: slots 0..3 <- sub-tile 2*st, slots 4..7 <- sub-tile 2*st+1
-    u32x4 pf[2];
-#pragma unroll
-    for (int st = 0; st < 2; ++st) {
-      pf[st][0] = Mma16<DT>::pack2(s[2 * st][0], s[2 * st][1]);
-      pf[st][1] = Mma16<DT>::pack2(s[2 * st][2], s[2 * st][3]);
-      pf[st][2] = Mma16<DT>::pack2(s[2 * st + 1][0], s[2 * st + 1][1]);
-      pf[st][3] = Mma16<DT>::pack2(s[2 * st + 1][2], s[2 * st + 1][3]);
-    }
+    // P^T as the B operand: slots 0..3 <- sub-tile 0, slots 4..7 <- sub-tile 1
+    u32x4 pf;
+    pf[0] = Mma16<DT>::pack2(s[0][0], s[0][1]);
+    pf[1] = Mma16<DT>::pack2(s[0][2], s[0][3]);
+    pf[2] = Mma16<DT>::pack2(s[1][0], s[1][1]);
+    pf[3] = Mma16<DT>::pack2(s[1][2], s[1][3]);
 
-    __syncthreads();  // V^T tile visible
     // ---- O^T += V^T . P^T ----
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int d = 16 * mt + c;
       const int sw = (mt & 3) << 1;
-#pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        const u32x4 a = *(const u32x4*)(vt + d * kVtRowBytes + (((4 * st + g) ^ sw) << 4));
-        o[mt] = Mma16<DT>::run(a, pf[st], o[mt]);
-      }
+      const u32x4 a = *(const u32x4*)(vt + d * kVtRowBytes + (((4 * st + g) ^ sw) << 4));
+      o[mt] = Mma16<DT>::run(a, pf, o[mt]);
+    }
+  };
+
+  HalfTile ha, hb;
+  load_half(k_begin, ha);
+  for (int t0 = k_begin; t0 < k_end; t0 += kTile) {
+    const bool second = t0 + 32 < k_end;
+    if (second) load_half(t0 + 32, hb);
+    __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic below
+    compute_half(t0, ha, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (second) {
+      if (t0 + kTile < k_end) load_half(t0 + kTile, ha);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_half(t0 + 32, hb, 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
@@ -416,7 +438,7 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   hipStream_t s = (hipStream_t)stream;
   const int units = Hkv * p.hchunks;
   const int wpb = pick_waves_per_block(units);
-  const dim3 grid1((uint32_t)p.nsplit_max, (uint32_t)(units / wpb), (uint32_t)B);
+  const dim3 grid1((uint32_t)(units / wpb), (uint32_t)p.nsplit_max, (uint32_t)B);
   const dim3 grid2((uint32_t)Hq, (uint32_t)B);
 #define DLB_LAUNCH_DECODE_W(DT_, D_, W_)                                                       \
   do {                                                                                         \
