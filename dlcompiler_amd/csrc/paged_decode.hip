@@ -7,9 +7,12 @@
 // the query heads of the group are batched against the head's K/V stream, online softmax in
 // fp32, P rounded to the cache dtype before P.V, split-KV partials (O, m, l) combined by a
 // second kernel -- with a different decomposition:
-//   * a work item is (sequence, kv head, KV chunk of `keys_per_split` tokens) instead of a
-//     fixed four-way split, so items are equally long whatever the context length;
-//   * one wavefront per item.  S^T = K.Q^T runs on 16x16x32 MFMA with the K rows loaded
+//   * the KV streams of all sequences are laid end to end (in units of 32 keys) and cut into
+//     equal pieces, one per team of wavefronts (one wavefront per kv-head unit), as many
+//     teams as fit on the chip at once: every wavefront streams the same number of bytes
+//     whatever the mix of context lengths, instead of a fixed four-way split per sequence.
+//     A piece that crosses a sequence boundary yields one partial per sequence;
+//   * one wavefront per (piece, kv-head unit).  S^T = K.Q^T runs on 16x16x32 MFMA with the K rows loaded
 //     straight from HBM into the A-operand layout (d is contiguous in memory and in the
 //     operand), so K never touches LDS;
 //   * V needs the key index contiguous per lane, so its tile is transposed on the way into
@@ -32,8 +35,9 @@ struct DecodeParams {
   void* o;
   const int32_t* block_table;
   const int32_t* kv_len;
-  float* ws_o;   // [B, Hq, nsplit_max, D]
-  float* ws_ml;  // [B, Hq, nsplit_max, 2]
+  float* ws_o;      // [B, Hq, nsplit_max, D]
+  float* ws_ml;     // [B, Hq, nsplit_max, 2]
+  int32_t* ws_np;   // [B] partials written for each sequence
   int64_t q_sb, q_sh;
   int64_t k_sp, k_st, k_sh;
   int64_t v_sp, v_st, v_sh;
@@ -42,7 +46,8 @@ struct DecodeParams {
   int B, Hq, Hkv, group, hchunks;
   int page, page_shift;  // page_shift < 0: page is not a power of two
   int max_blocks;
-  int keys_per_split, nsplit_max;
+  int min_units, nsplit_max;  // smallest piece (32-key units); partial slots per (sequence, head)
+  int num_teams;
   float scale_log2e;
   float sm_scale;
   int window;      // > 0: keys older than (ctx - 1 - window) are masked (paged_attention.py:163-167)
@@ -81,47 +86,58 @@ struct Mma16<DLB_DTYPE_F16> {
 constexpr int kTile = 64;          // keys per iteration
 constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
 
-// WPB wavefronts per workgroup: wave w handles (kv head, head chunk) unit blockIdx.y * WPB + w
-// of the SAME (sequence, KV chunk), so the waves of a workgroup read neighbouring 256-byte
-// head slices of the same token rows at the same time (whole 2 KB token rows in flight).
 template <int DT, int D, int WPB, bool POW2>
 __global__ __launch_bounds__(64 * WPB, 2) void paged_decode_split_kernel(const DecodeParams p) {
   constexpr int KS = D / 32;   // MFMA k-steps over the head dim
   constexpr int MT = D / 16;   // 16-row tiles of O^T
   constexpr int DG = D / 8;    // 8-dim groups per key row
+  static_assert(WPB == 1, "one wavefront per workgroup");
 
-  // grid: x = (kv head, head chunk) unit, y = KV chunk, z = sequence.  The unit is the fastest
-  // index, so workgroups that start together read the 256-byte head slices of the SAME token
-  // rows at the same time: whole 2 KB cache rows are in flight together and DRAM pages are hit
-  // while open.
-  const int split = blockIdx.y;
-  const int wave = threadIdx.x >> 6;
-  const int unit = blockIdx.x * WPB + wave;
+  // grid: x = (kv head, head chunk) unit, y = team.  The unit is the fastest index, so the
+  // wavefronts that start together read the 256-byte head slices of the SAME token rows at the
+  // same time: whole 2 KB cache rows are in flight together and DRAM pages are hit while open.
+  const int wave = 0;
+  const int unit = blockIdx.x;
+  const int team = blockIdx.y;
   const int kvh = unit / p.hchunks;
   const int hchunk = unit - kvh * p.hchunks;
-  const int b = blockIdx.z;
-  const int ctx = p.kv_len[b];
-  const int kv_min = p.window > 0 ? max(ctx - 1 - p.window, 0) : 0;  // first visible key
-  int k_begin = split * p.keys_per_split;
-  if (k_begin >= ctx) return;  // uniform for the wave; also covers ctx <= 0
-  const int k_end = min(ctx, k_begin + p.keys_per_split);
-  if (k_end <= kv_min) return;  // chunk entirely outside the sliding window
-  k_begin = max(k_begin, kv_min & ~(kTile - 1));  // start at the tile that holds kv_min
 
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;  // lane group 0..3
   const int c = lane & 15;  // column (query head) / row (key) inside a 16-tile
 
   __shared__ __attribute__((aligned(16))) unsigned char vt_all[WPB][D * kVtRowBytes];
+  __shared__ int32_t seg_lds[2][64];  // (first unit, units) of the 64 sequences being walked
   unsigned char* vt = vt_all[wave];
 
   const unsigned short* qb = (const unsigned short*)p.q;
-  const int32_t* bt = p.block_table + (int64_t)b * p.bt_stride;
-
-  // Q^T as the B operand: lane (n = query head c, k = dims 32*ks + 8g .. +8)
   const int hq_local = hchunk * 16 + c;
   const bool head_ok = hq_local < p.group;
   const int head = kvh * p.group + hq_local;
+
+  // ---- this team's piece of the concatenated KV streams (32-key units) ----
+  auto units_of = [&](int bb) { return bb < p.B ? (max(p.kv_len[bb], 0) + 31) >> 5 : 0; };
+  int total = 0;
+  for (int b0 = 0; b0 < p.B; b0 += 64) {
+    int t = units_of(b0 + lane);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) t += __shfl_xor(t, d);
+    total += t;
+  }
+  const int upt = max((total + p.num_teams - 1) / p.num_teams, p.min_units);  // units per team
+  const int lo = team * upt;
+  if (lo >= total) return;
+  const int hi = min(lo + upt, total);
+
+  // one sequence segment [k_begin, k_end) of sequence b -> partial number `piece` of b
+  auto process_segment = [&](int b, int k_begin, int k_end, int piece) {
+  const int ctx = p.kv_len[b];
+  k_end = min(k_end, ctx);
+  const int kv_min = p.window > 0 ? max(ctx - 1 - p.window, 0) : 0;  // first visible key
+  k_begin = max(k_begin, kv_min & ~31);  // start at the half tile that holds kv_min
+  const int32_t* bt = p.block_table + (int64_t)b * p.bt_stride;
+
+  // Q^T as the B operand: lane (n = query head c, k = dims 32*ks + 8g .. +8)
   u32x4 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -280,7 +296,7 @@ __global__ __launch_bounds__(64 * WPB, 2) void paged_decode_split_kernel(const D
   };
 
   HalfTile ha, hb;
-  load_half(k_begin, ha);
+  if (k_begin < k_end) load_half(k_begin, ha);  // (a segment entirely before the window is empty)
   for (int t0 = k_begin; t0 < k_end; t0 += kTile) {
     const bool second = t0 + 32 < k_end;
     if (second) load_half(t0 + 32, hb);
@@ -299,56 +315,120 @@ __global__ __launch_bounds__(64 * WPB, 2) void paged_decode_split_kernel(const D
   l_run += __shfl_xor(l_run, 32);
 
   if (head_ok) {
-    const int64_t slot = ((int64_t)b * p.Hq + head) * p.nsplit_max + split;
+    const int64_t slot = ((int64_t)b * p.Hq + head) * p.nsplit_max + piece;
     float* wo = p.ws_o + slot * D;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *(f32x4*)(wo + 16 * mt + 4 * g) = o[mt];
     if (g == 0) {
-      p.ws_ml[slot * 2 + 0] = m_run;
+      p.ws_ml[slot * 2 + 0] = m_run;  // -inf with l = 0 for an empty segment: weight 0 in the combine
       p.ws_ml[slot * 2 + 1] = l_run;
     }
   }
+  };  // process_segment
+
+  // ---- walk the sequences this piece overlaps ----
+  int carry = 0;  // units of all sequences before b0
+  for (int b0 = 0; b0 < p.B; b0 += 64) {
+    const int t = units_of(b0 + lane);
+    int incl = t;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    const int excl = carry + incl - t;
+    uint64_t hit = __ballot(t > 0 && excl < hi && excl + t > lo);
+    // park the per-sequence values in LDS: nothing per-lane stays live across a segment
+    seg_lds[0][lane] = excl;
+    seg_lds[1][lane] = t;
+    carry = __builtin_amdgcn_readfirstlane(carry + __shfl(incl, 63));
+    while (hit) {  // wave-uniform
+      const int l = __builtin_ctzll(hit);
+      hit &= hit - 1;
+      const int b = b0 + l;
+      const int pb = __builtin_amdgcn_readfirstlane(seg_lds[0][l]);
+      const int tb = __builtin_amdgcn_readfirstlane(seg_lds[1][l]);
+      const int first_team = pb / upt;
+      if (team == first_team && unit == 0 && lane == 0)
+        p.ws_np[b] = (pb + tb - 1) / upt - first_team + 1;
+      process_segment(b, (max(lo, pb) - pb) * 32, (min(hi, pb + tb) - pb) * 32, team - first_team);
+    }
+    if (carry >= hi) break;
+  }
 }
 
-// Combine the split partials: O = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s
-// (paged_attention.py:238-285 with the exponent in base 2).
+// Combine the partials of one (sequence, head): O = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s
+// (paged_attention.py:238-285 with the exponent in base 2).  Lane s of every wave fetches
+// (m_s, l_s) so the weights come from two wave reductions; the O_s rows are then read with all
+// loads of a group of four in flight.
 template <int DT, int D>
 __global__ __launch_bounds__(D) void paged_decode_combine_kernel(const DecodeParams p) {
   const int head = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int lane = d & 63;
   const int ctx = p.kv_len[b];
   float acc = 0.0f;
   if (ctx > 0) {
-    const int ns = (ctx + p.keys_per_split - 1) / p.keys_per_split;
-    // chunks entirely before the sliding window were skipped by the split kernel
-    const int s0 = p.window > 0 ? max(ctx - 1 - p.window, 0) / p.keys_per_split : 0;
+    const int ns = p.ws_np[b];  // pieces of this sequence (empty ones carry m = -inf, l = 0)
     const int64_t slot0 = ((int64_t)b * p.Hq + head) * p.nsplit_max;
     float m = -__builtin_inff();
-    for (int s = s0; s < ns; ++s) m = fmaxf(m, p.ws_ml[(slot0 + s) * 2]);
+    for (int s0 = 0; s0 < ns; s0 += 64) {
+      float ms = (s0 + lane < ns) ? p.ws_ml[(slot0 + s0 + lane) * 2] : -__builtin_inff();
+#pragma unroll
+      for (int x = 32; x >= 1; x >>= 1) ms = fmaxf(ms, __shfl_xor(ms, x));
+      m = fmaxf(m, ms);
+    }
     float den = 0.0f;
-    for (int s = s0; s < ns; ++s) {
-      const float w = __builtin_amdgcn_exp2f(p.ws_ml[(slot0 + s) * 2] - m);
-      den += w * p.ws_ml[(slot0 + s) * 2 + 1];
-      acc += w * p.ws_o[(slot0 + s) * D + d];
+    for (int s0 = 0; s0 < ns; s0 += 64) {
+      const bool live = s0 + lane < ns;
+      const float w = live ? __builtin_amdgcn_exp2f(p.ws_ml[(slot0 + s0 + lane) * 2] - m) : 0.0f;
+      float wl = live ? w * p.ws_ml[(slot0 + s0 + lane) * 2 + 1] : 0.0f;
+#pragma unroll
+      for (int x = 32; x >= 1; x >>= 1) wl += __shfl_xor(wl, x);
+      den += wl;
+      const int n = min(64, ns - s0);
+      for (int s = 0; s < n; s += 4) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = (s + u < n) ? p.ws_o[(slot0 + s0 + s + u) * D + d] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc += __shfl(w, min(s + u, 63)) * v[u];
+      }
     }
     acc /= den;
   }
   Elem<DT>::store1(p.o, (int64_t)b * p.o_sb + (int64_t)head * p.o_sh + d, acc);
 }
 
-int pick_keys_per_split(int B, int Hkv, int hchunks, int max_ctx) {
-  // enough work items to cover the chip several times over, but no smaller than 2 tiles
+// smallest piece a team may get, in 32-key units: 512 keys, less for small problems so that
+// the chip still sees a few thousand wavefronts
+int pick_min_units(int B, int Hkv, int hchunks, int max_ctx) {
   const int64_t units = (int64_t)B * Hkv * hchunks;
   int kps = 512;
-  if (const char* env = getenv("DLB_DECODE_KPS")) kps = atoi(env);
   while (kps > 128 && units * ((max_ctx + kps - 1) / kps) < 4096) kps >>= 1;
-  return kps;
+  return kps / 32;
 }
 
-int pick_waves_per_block(int units) {
-  int wpb = 1;
-  if (const char* env = getenv("DLB_DECODE_WPB")) wpb = atoi(env);
-  while (wpb > 1 && units % wpb != 0) wpb >>= 1;
-  return wpb;
+// partial slots per (sequence, head): a sequence of T units cut into pieces of >= min_units
+// overlaps at most T / min_units + 2 of them
+int partial_slots(int max_ctx, int min_units) {
+  const int t = (max_ctx + 31) / 32;
+  return t / min_units + 2;
+}
+
+// teams that are resident together: 8 wavefronts per CU (2 per SIMD) / wavefronts per team
+int pick_num_teams(int units_per_team) {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  int mult = 1;
+  if (const char* env = getenv("DLB_DECODE_TEAM_MULT")) mult = atoi(env);
+  return max(1, cus * 8 * mult / units_per_team);
 }
 
 }  // namespace
@@ -361,9 +441,8 @@ extern "C" size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int p
   const int hchunks = (group + 15) / 16;
   const int64_t max_ctx = (int64_t)page * max_blocks;
   if (max_ctx > 0x7fffffff) return 0;
-  const int kps = dlb::pick_keys_per_split(B, Hkv, hchunks, (int)max_ctx);
-  const int64_t ns = (max_ctx + kps - 1) / kps;
-  return (size_t)B * Hq * ns * (D + 2) * sizeof(float);
+  const int64_t ns = dlb::partial_slots((int)max_ctx, dlb::pick_min_units(B, Hkv, hchunks, (int)max_ctx));
+  return (size_t)B * Hq * ns * (D + 2) * sizeof(float) + (size_t)B * sizeof(int32_t);
 }
 
 extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache,
@@ -426,36 +505,31 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
     if ((1 << sh) == page) p.page_shift = sh;
   p.max_blocks = max_blocks;
   const int max_ctx = page * max_blocks;
-  p.keys_per_split = pick_keys_per_split(B, Hkv, p.hchunks, max_ctx);
-  p.nsplit_max = (max_ctx + p.keys_per_split - 1) / p.keys_per_split;
+  p.min_units = pick_min_units(B, Hkv, p.hchunks, max_ctx);
+  p.nsplit_max = partial_slots(max_ctx, p.min_units);
   p.scale_log2e = sm_scale * 1.4426950408889634f;
   p.sm_scale = sm_scale;
   p.window = window_size;
   p.softcap = logit_softcapping;
   p.ws_o = (float*)ws;
   p.ws_ml = p.ws_o + (size_t)B * Hq * p.nsplit_max * D;
+  p.ws_np = (int32_t*)(p.ws_ml + (size_t)B * Hq * p.nsplit_max * 2);
 
   hipStream_t s = (hipStream_t)stream;
   const int units = Hkv * p.hchunks;
-  const int wpb = pick_waves_per_block(units);
-  const dim3 grid1((uint32_t)(units / wpb), (uint32_t)p.nsplit_max, (uint32_t)B);
+  p.num_teams = pick_num_teams(units);
+  if (units > 65535 || p.num_teams > 65535) return DLB_ERR_UNSUPPORTED;
+  const dim3 grid1((uint32_t)units, (uint32_t)p.num_teams);
   const dim3 grid2((uint32_t)Hq, (uint32_t)B);
-#define DLB_LAUNCH_DECODE_W(DT_, D_, W_)                                                       \
-  do {                                                                                         \
-    if (p.page_shift >= 0)                                                                     \
-      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, W_, true>), grid1, dim3(64 * W_), \
-                         0, s, p);                                                             \
-    else                                                                                       \
-      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, W_, false>), grid1,               \
-                         dim3(64 * W_), 0, s, p);                                              \
-  } while (0)
-#define DLB_LAUNCH_DECODE(DT_, D_)                                                              \
-  do {                                                                                          \
-    if (wpb == 8) DLB_LAUNCH_DECODE_W(DT_, D_, 8);                                              \
-    else if (wpb == 4) DLB_LAUNCH_DECODE_W(DT_, D_, 4);                                         \
-    else if (wpb == 2) DLB_LAUNCH_DECODE_W(DT_, D_, 2);                                         \
-    else DLB_LAUNCH_DECODE_W(DT_, D_, 1);                                                       \
-    hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p);       \
+#define DLB_LAUNCH_DECODE(DT_, D_)                                                          \
+  do {                                                                                      \
+    if (p.page_shift >= 0)                                                                  \
+      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, 1, true>), grid1, dim3(64), 0, \
+                         s, p);                                                             \
+    else                                                                                    \
+      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, 1, false>), grid1, dim3(64),   \
+                         0, s, p);                                                          \
+    hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p);   \
   } while (0)
   if (dtype == DLB_DTYPE_BF16) {
     if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 128);
@@ -464,7 +538,6 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
     if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
     else DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 64);
   }
-#undef DLB_LAUNCH_DECODE_W
 #undef DLB_LAUNCH_DECODE
   return launch_status();
 }
