@@ -193,6 +193,10 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
  *   hq [num_mblocks * block_m, I] fp8 and hs [num_mblocks * block_m, I/128]: row r holds
  *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r
  * H % 128 == 0, I % 128 == 0.
+ * block_m selects the kernel: 64 = four-wave tiles of 64 rows, weights streamed straight into
+ * operand registers (fastest with w_layout 1); 128 = eight-wave tiles of 128 rows x 256
+ * columns with both operands staged by direct-to-LDS loads (reads row-major weights, w_layout
+ * 0, at full efficiency; hq/out must be 16-byte aligned).
  * w_layout selects how the fp8 weight bytes of both GEMMs are stored:
  *   0  row-major [E, N, K] (the reference's w1/w2 layout);
  *   1  MFMA-operand order, a one-time re-arrangement done when the weights are loaded: for
