@@ -79,6 +79,22 @@ def test_logit_softcapping(dev, cap):
     _run_case(dev, [300, 2000], 8, 2, 64, 16, torch.float16, softcap=cap, window=100)
 
 
+def test_many_short_sequences(dev):
+    # more sequences than lanes in a wavefront and contexts far shorter than a work piece: a
+    # piece then spans many sequences and the per-sequence scan walks several blocks of 64
+    gen = torch.Generator().manual_seed(11)
+    lens = torch.randint(0, 70, (150,), generator=gen).tolist()
+    lens[0], lens[64], lens[149] = 1, 0, 33
+    _run_case(dev, lens, 8, 2, 128, 16, torch.bfloat16, seed=4)
+    _run_case(dev, lens[:131], 4, 4, 64, 32, torch.float16, seed=5, window=20)
+
+
+def test_one_long_sequence_many_pieces(dev):
+    # a single long context is cut into many pieces (one partial each)
+    _run_case(dev, [20000], 8, 2, 128, 64, torch.bfloat16, seed=6)
+    _run_case(dev, [3, 20000, 5], 8, 8, 64, 16, torch.float16, seed=7, window=3000)
+
+
 def test_non_power_of_two_page_and_spare_pages(dev):
     _run_case(dev, [700, 48, 49, 1], 8, 2, 128, 48, torch.bfloat16, num_pages=64)
 
