@@ -101,6 +101,26 @@ def current_stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device):
+    """Context that makes ``device`` current for the launch; free when it already is."""
+    import torch
+
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
 def require_cuda(*tensors) -> None:
     for t in tensors:
         if t is not None and not t.is_cuda:

@@ -21,8 +21,6 @@
 //     registers ARE the B operand of O^T = V^T.P^T: P never moves between lanes.
 // The kernel is an HBM stream (4 FLOP/byte at GQA 4:1); everything else is sized to keep
 // tens of KB of loads in flight per CU.
-#include <stdlib.h>
-
 #include "common.h"
 
 namespace dlb {
@@ -86,17 +84,15 @@ struct Mma16<DLB_DTYPE_F16> {
 constexpr int kTile = 64;          // keys per iteration
 constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
 
-template <int DT, int D, int WPB, bool POW2>
-__global__ __launch_bounds__(64 * WPB, 2) void paged_decode_split_kernel(const DecodeParams p) {
+template <int DT, int D, bool POW2>
+__global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeParams p) {
   constexpr int KS = D / 32;   // MFMA k-steps over the head dim
   constexpr int MT = D / 16;   // 16-row tiles of O^T
   constexpr int DG = D / 8;    // 8-dim groups per key row
-  static_assert(WPB == 1, "one wavefront per workgroup");
 
   // grid: x = (kv head, head chunk) unit, y = team.  The unit is the fastest index, so the
   // wavefronts that start together read the 256-byte head slices of the SAME token rows at the
   // same time: whole 2 KB cache rows are in flight together and DRAM pages are hit while open.
-  const int wave = 0;
   const int unit = blockIdx.x;
   const int team = blockIdx.y;
   const int kvh = unit / p.hchunks;
@@ -106,9 +102,8 @@ __global__ __launch_bounds__(64 * WPB, 2) void paged_decode_split_kernel(const D
   const int g = lane >> 4;  // lane group 0..3
   const int c = lane & 15;  // column (query head) / row (key) inside a 16-tile
 
-  __shared__ __attribute__((aligned(16))) unsigned char vt_all[WPB][D * kVtRowBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char vt[D * kVtRowBytes];  // this wave's V^T tile
   __shared__ int32_t seg_lds[2][64];  // (first unit, units) of the 64 sequences being walked
-  unsigned char* vt = vt_all[wave];
 
   const unsigned short* qb = (const unsigned short*)p.q;
   const int hq_local = hchunk * 16 + c;
@@ -426,9 +421,7 @@ int pick_num_teams(int units_per_team) {
     else
       cus = 256;
   }
-  int mult = 1;
-  if (const char* env = getenv("DLB_DECODE_TEAM_MULT")) mult = atoi(env);
-  return max(1, cus * 8 * mult / units_per_team);
+  return max(1, cus * 8 / units_per_team);
 }
 
 }  // namespace
@@ -524,10 +517,10 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
 #define DLB_LAUNCH_DECODE(DT_, D_)                                                          \
   do {                                                                                      \
     if (p.page_shift >= 0)                                                                  \
-      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, 1, true>), grid1, dim3(64), 0, \
+      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, true>), grid1, dim3(64), 0, \
                          s, p);                                                             \
     else                                                                                    \
-      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, 1, false>), grid1, dim3(64),   \
+      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, false>), grid1, dim3(64),   \
                          0, s, p);                                                          \
     hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p);   \
   } while (0)

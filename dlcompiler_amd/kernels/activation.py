@@ -29,7 +29,7 @@ def silu_and_mul(gate_up: torch.Tensor, out: torch.Tensor = None):
         res = out.new_empty((M, N))
     if M > 0 and N > 0:
         lib = _lib.load()
-        with torch.cuda.device(gate_up.device):
+        with _lib.device_guard(gate_up.device):
             st = lib.dlb_silu_and_mul(gate_up.data_ptr(), res.data_ptr(), M, N,
                                       gate_up.stride(0) if M > 1 else 2 * N,
                                       res.stride(0) if M > 1 else N,

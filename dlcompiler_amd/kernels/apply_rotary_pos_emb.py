@@ -42,7 +42,7 @@ def apply_rotary_pos_emb(
     if seq_len == 0:
         return q_embed, k_embed
     lib = _lib.load()
-    with torch.cuda.device(q.device):
+    with _lib.device_guard(q.device):
         st = lib.dlb_apply_rotary_pos_emb(
             q.data_ptr(), k.data_ptr(), cos2.data_ptr(), sin2.data_ptr(), q_embed.data_ptr(),
             k_embed.data_ptr(), seq_len, q.size(1), k.size(1), D, q.stride(0), q.stride(1),

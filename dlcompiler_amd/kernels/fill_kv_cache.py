@@ -39,7 +39,7 @@ def fill_kv_cache(
     lib = _lib.load()
     # converted copies must stay referenced until the launch is enqueued
     q_start_i, q_len_i, kv_len_i = _i32(q_start_loc), _i32(q_seq_length), _i32(kv_seq_length)
-    with torch.cuda.device(k_states.device):
+    with _lib.device_guard(k_states.device):
         st = lib.dlb_fill_kv_cache(
             k_states.data_ptr(), v_states.data_ptr(), k_caches.data_ptr(), v_caches.data_ptr(),
             q_start_i.data_ptr(), q_len_i.data_ptr(), kv_len_i.data_ptr(),

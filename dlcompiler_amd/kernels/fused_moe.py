@@ -34,7 +34,7 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
     xs = torch.empty((M, K // 128), dtype=torch.float32, device=x.device)
     if M > 0:
         lib = _lib.load()
-        with torch.cuda.device(x.device):
+        with _lib.device_guard(x.device):
             st = lib.dlb_per_token_group_quant_fp8(
                 x.data_ptr(), xq.data_ptr(), xs.data_ptr(), M, K, x.stride(0) if M > 1 else K, K,
                 K // 128, _lib.torch_dtype_code(x.dtype), _lib.current_stream_ptr(x.device))
@@ -133,7 +133,7 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
 
     lib = _lib.load()
     stream = _lib.current_stream_ptr(dev)
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         hook("gate_up")
         st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
                                           w1_s.data_ptr(), sorted_ids.data_ptr(),
@@ -202,7 +202,7 @@ def fused_moe(hidden_states: torch.Tensor,
     lib = _lib.load()
     code = _lib.torch_dtype_code(dt)
     stream = _lib.current_stream_ptr(dev)
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         st = lib.dlb_moe_gemm_16bit_gate_up(hidden_states.data_ptr(), w1.data_ptr(),
                                             sorted_ids.data_ptr(), expert_ids.data_ptr(),
                                             num_mblocks, _ALIGN_BLOCK, M, topk, H, I,

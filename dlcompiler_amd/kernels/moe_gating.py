@@ -31,7 +31,7 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True):
     ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
     if T > 0:
         lib = _lib.load()
-        with torch.cuda.device(logits.device):
+        with _lib.device_guard(logits.device):
             st = lib.dlb_moe_topk_softmax_f32(logits.data_ptr(), weights.data_ptr(),
                                               ids.data_ptr(), T, E, k,
                                               logits.stride(0) if T > 1 else E,
@@ -66,18 +66,21 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     dev = ids.device
     cap = numel + num_experts * (block_size - 1)
     nblk = max(1, -(-cap // block_size))
-    sorted_ids = torch.empty((cap,), dtype=torch.int32, device=dev)
-    expert_ids = torch.empty((nblk,), dtype=torch.int32, device=dev)
-    num_post = torch.empty((1,), dtype=torch.int32, device=dev)
-    counts = torch.empty((num_experts,), dtype=torch.int32, device=dev)
     lib = _lib.load()
-    ws_bytes = lib.dlb_moe_align_ws_bytes(numel, num_experts)
-    ws = torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    ws_words = max((lib.dlb_moe_align_ws_bytes(numel, num_experts) + 3) // 4, 1)
+    # one allocation, carved into the four results and the scratch (16-byte aligned pieces)
+    sizes = (cap, nblk, 1, num_experts, ws_words)
+    offs, total = [], 0
+    for n in sizes:
+        offs.append(total)
+        total += (n + 3) & ~3
+    buf = torch.empty((total,), dtype=torch.int32, device=dev)
+    sorted_ids, expert_ids, num_post, counts, ws = (buf[o:o + n] for o, n in zip(offs, sizes))
+    with _lib.device_guard(dev):
         st = lib.dlb_moe_align_block_size(ids.data_ptr(), numel, num_experts, block_size,
                                           sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk,
                                           counts.data_ptr(), num_post.data_ptr(), ws.data_ptr(),
-                                          ws.numel(), _lib.current_stream_ptr(dev))
+                                          ws.numel() * 4, _lib.current_stream_ptr(dev))
     _lib.check(st, "dlb_moe_align_block_size")
     if return_counts:
         return sorted_ids, expert_ids, num_post, counts

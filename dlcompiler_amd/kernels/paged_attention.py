@@ -68,7 +68,7 @@ def paged_attention_fwd(
         assert q.dim() == 3 and o.dim() == 3
         q_start_loc = _as_int32(q_start_loc).contiguous()
         q_seqlens = _as_int32(q_seqlens).contiguous()
-        with torch.cuda.device(q.device):
+        with _lib.device_guard(q.device):
             st = lib.dlb_paged_prefill_attn(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), block_offsets.data_ptr(),
                 q_start_loc.data_ptr(), q_seqlens.data_ptr(), kv_seqlens.data_ptr(), batch, head,
@@ -85,7 +85,7 @@ def paged_attention_fwd(
     assert o3.data_ptr() == o.data_ptr()
     ws_bytes = lib.dlb_paged_decode_ws_bytes(batch, head, num_kv_heads, Lq, page, max_blocks)
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=q.device)
-    with torch.cuda.device(q.device):
+    with _lib.device_guard(q.device):
         st = lib.dlb_paged_decode_attn(
             q3.data_ptr(), k.data_ptr(), v.data_ptr(), o3.data_ptr(), block_offsets.data_ptr(),
             kv_seqlens.data_ptr(), batch, head, num_kv_heads, Lq, page, max_blocks,

@@ -34,7 +34,7 @@ def context_attention_fwd(q, k, v, o, b_start_loc, b_seq_len, max_input_len):
     lib = _lib.load()
     start = _as_int32(b_start_loc)
     lens = _as_int32(b_seq_len)
-    with torch.cuda.device(q.device):
+    with _lib.device_guard(q.device):
         st = lib.dlb_prefill_attn_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), start.data_ptr(),
             lens.data_ptr(), batch, head, k.shape[1], Lq, int(max_input_len),

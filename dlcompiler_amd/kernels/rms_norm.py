@@ -35,7 +35,7 @@ def rms_norm(
     weight = weight.contiguous()
     if residual is None:
         if seq_len > 0:
-            with torch.cuda.device(hidden_states.device):
+            with _lib.device_guard(hidden_states.device):
                 st = lib.dlb_rms_norm(x2.data_ptr(), weight.data_ptr(), None, o2.data_ptr(), None,
                                       seq_len, feat_size, x2.stride(0), 0, o2.stride(0), 0,
                                       float(eps), code, stream)
@@ -48,7 +48,7 @@ def rms_norm(
     r2 = residual.view(seq_len, feat_size)
     or2 = out_residual.view(seq_len, feat_size)
     if seq_len > 0:
-        with torch.cuda.device(hidden_states.device):
+        with _lib.device_guard(hidden_states.device):
             st = lib.dlb_rms_norm(x2.data_ptr(), weight.data_ptr(), r2.data_ptr(), o2.data_ptr(),
                                   or2.data_ptr(), seq_len, feat_size, x2.stride(0), r2.stride(0),
                                   o2.stride(0), or2.stride(0), float(eps), code, stream)
