@@ -369,13 +369,17 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
     if cpu:
         from oracle import fused_moe as ofm
 
-        n = 64
+        # the whole workload, repeated: about ten seconds of CPU work on the box's 16 cores
+        ofm.fused_moe_fp8(x_cpu[:64], w1q, w1s, w2q, w2s, tw_cpu[:64], ids_cpu[:64])  # warm-up
+        reps = 0
         t0 = time.perf_counter()
-        ofm.fused_moe_fp8(x_cpu[:n], w1q, w1s, w2q, w2s, tw_cpu[:n], ids_cpu[:n])
-        dt = time.perf_counter() - t0
-        res["cpu_baseline"] = {"value": flops * n / T / dt / 1e12, "unit": "TFLOP/s",
+        while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 40):
+            ofm.fused_moe_fp8(x_cpu, w1q, w1s, w2q, w2s, tw_cpu, ids_cpu)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": flops / dt / 1e12, "unit": "TFLOP/s",
                                "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": f"first {n} of {T} tokens (all 64 experts de-quantised), 1 rep"}
+                               "sample": f"all {T} tokens, {reps} reps ({dt * reps:.1f} s of CPU time)"}
     return res
 
 
