@@ -12,7 +12,19 @@ import torch
 from .. import _lib
 from .moe_gating import moe_align_block_size
 
-_ALIGN_BLOCK = int(__import__('os').environ.get('DLB_MOE_BLOCK', '64'))  # rows per grouped-GEMM workgroup tile
+import os
+
+_BLOCK_OVERRIDE = int(os.environ.get("DLB_MOE_BLOCK", "0"))  # 64 / 128 force a tile height
+
+
+def _align_block(weights_shuffled: bool) -> int:
+    """Rows per grouped-GEMM workgroup tile = alignment block of the routing.  Row-major
+    weights (the reference layout) run fastest on the 128-row kernel, which stages them through
+    LDS a full cache line per row; operand-order weights on the 64-row kernel, which streams
+    them straight into MFMA operand registers."""
+    if _BLOCK_OVERRIDE in (64, 128):
+        return _BLOCK_OVERRIDE
+    return 64 if weights_shuffled else 128
 
 
 def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
@@ -118,13 +130,14 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     w2_s = w2_s.to(torch.float32).contiguous()
 
     hook("align")
-    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, _ALIGN_BLOCK, num_experts)
+    block = _align_block(weights_shuffled)
+    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, block, num_experts)
     num_mblocks = expert_ids.numel()
     hook("quant")
     xq, xs = per_token_group_quant_fp8(hidden_states)
     hook("alloc")
 
-    rows = num_mblocks * _ALIGN_BLOCK
+    rows = num_mblocks * block
     hq = torch.empty((rows, I), dtype=torch.float8_e4m3fn, device=dev)
     hs = torch.empty((rows, I // 128), dtype=torch.float32, device=dev)
     full = (expert_offset == 0 and num_experts == E)
@@ -137,7 +150,7 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
         hook("gate_up")
         st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
                                           w1_s.data_ptr(), sorted_ids.data_ptr(),
-                                          expert_ids.data_ptr(), num_mblocks, _ALIGN_BLOCK, T, topk,
+                                          expert_ids.data_ptr(), num_mblocks, block, T, topk,
                                           H, I, expert_offset, E, int(weights_shuffled),
                                           hq.data_ptr(), hs.data_ptr(), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_gate_up")
@@ -145,7 +158,7 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
         st = lib.dlb_moe_gemm_fp8_down(hq.data_ptr(), hs.data_ptr(), w2_q.data_ptr(),
                                        w2_s.data_ptr(), sorted_ids.data_ptr(),
                                        expert_ids.data_ptr(), topk_weights.data_ptr(),
-                                       num_mblocks, _ALIGN_BLOCK, T, topk, H, I, expert_offset, E,
+                                       num_mblocks, block, T, topk, H, I, expert_offset, E,
                                        int(weights_shuffled),
                                        slots.data_ptr(), _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_down")
@@ -193,9 +206,10 @@ def fused_moe(hidden_states: torch.Tensor,
         topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
     topk_weights = topk_weights.to(torch.float32).contiguous()
 
-    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, _ALIGN_BLOCK, num_experts)
+    block = _align_block(weights_shuffled)
+    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, block, num_experts)
     num_mblocks = expert_ids.numel()
-    act = torch.empty((num_mblocks * _ALIGN_BLOCK, I), dtype=dt, device=dev)
+    act = torch.empty((num_mblocks * block, I), dtype=dt, device=dev)
     full = (expert_offset == 0 and num_experts == E)
     slots = (torch.empty if full else torch.zeros)((M * topk, H), dtype=dt, device=dev)
     out = torch.empty((M, H), dtype=dt, device=dev)
@@ -205,13 +219,13 @@ def fused_moe(hidden_states: torch.Tensor,
     with _lib.device_guard(dev):
         st = lib.dlb_moe_gemm_16bit_gate_up(hidden_states.data_ptr(), w1.data_ptr(),
                                             sorted_ids.data_ptr(), expert_ids.data_ptr(),
-                                            num_mblocks, _ALIGN_BLOCK, M, topk, H, I,
+                                            num_mblocks, block, M, topk, H, I,
                                             expert_offset, E, int(weights_shuffled),
                                             act.data_ptr(), code, stream)
         _lib.check(st, "dlb_moe_gemm_16bit_gate_up")
         st = lib.dlb_moe_gemm_16bit_down(act.data_ptr(), w2.data_ptr(), sorted_ids.data_ptr(),
                                          expert_ids.data_ptr(), topk_weights.data_ptr(),
-                                         num_mblocks, _ALIGN_BLOCK, M, topk, H, I, expert_offset,
+                                         num_mblocks, block, M, topk, H, I, expert_offset,
                                          E, int(weights_shuffled), slots.data_ptr(), code, stream)
         _lib.check(st, "dlb_moe_gemm_16bit_down")
         st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), M, topk, H, code, stream)

@@ -39,23 +39,30 @@ def test_reference_case(dev):
 @pytest.mark.parametrize("T,H,I,E,k", [(256, 256, 128, 8, 2), (1, 128, 128, 4, 1),
                                        (333, 512, 384, 64, 6), (512, 2048, 1408, 8, 6)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_fused_moe_parity(dev, T, H, I, E, k, dtype):
-    from dlcompiler_amd.kernels.fused_moe import fused_moe, shuffle_moe_weight
+def test_fused_moe_parity(dev, T, H, I, E, k, dtype, monkeypatch):
+    from dlcompiler_amd.kernels import fused_moe as fm
 
     x, w1, w2, tw, ids = _inputs(T, H, I, E, k, 1, dtype)
     args = (x.to(dev), w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev))
-    out = fused_moe(*args, k, renormalize=True)
     ref = ofm.fused_moe(x, w1, w2, tw, ids, renormalize=True)
-    assert out.shape == (T, H) and out.dtype == dtype
-    # north-star tolerance for 16-bit outputs: 2e-2 abs/rel, the absolute part taken relative
-    # to the output scale (a slot value's 16-bit rounding is proportional to its magnitude)
     scale = max(1.0, ref.float().abs().max().item())
-    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2 * scale)
-    err = ((out.cpu().double() - ref.double()).norm() / ref.double().norm()).item()
-    assert err < 5e-3
-    out2 = fused_moe(args[0], shuffle_moe_weight(args[1]), shuffle_moe_weight(args[2]), args[3],
-                     args[4], k, renormalize=True, weights_shuffled=True)
-    assert torch.equal(out2, out)
+
+    def check(out):
+        assert out.shape == (T, H) and out.dtype == dtype
+        # north-star tolerance for 16-bit outputs: 2e-2 abs/rel, the absolute part taken relative
+        # to the output scale (a slot value's 16-bit rounding is proportional to its magnitude)
+        torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2 * scale)
+        err = ((out.cpu().double() - ref.double()).norm() / ref.double().norm()).item()
+        assert err < 5e-3
+
+    check(fm.fused_moe(*args, k, renormalize=True))     # default tile height for row-major weights
+    for block in (64, 128):                              # both kernels, both weight layouts
+        monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+        out = fm.fused_moe(*args, k, renormalize=True)
+        check(out)
+        out2 = fm.fused_moe(args[0], fm.shuffle_moe_weight(args[1]), fm.shuffle_moe_weight(args[2]),
+                            args[3], args[4], k, renormalize=True, weights_shuffled=True)
+        assert torch.equal(out2, out)
 
 
 def test_expert_shard(dev):

@@ -53,20 +53,25 @@ def _check(out, ref):
                                        (1, 256, 256, 8, 2), (333, 512, 384, 64, 6),
                                        (64, 128, 128, 2, 1)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_fused_moe_fp8_parity(dev, T, H, I, E, k, dtype):
-    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8, shuffle_moe_weight_fp8
+def test_fused_moe_fp8_parity(dev, T, H, I, E, k, dtype, monkeypatch):
+    from dlcompiler_amd.kernels import fused_moe as fm
 
     x, w1q, w1s, w2q, w2s, tw, ids = _inputs(T, H, I, E, k, 1, dtype)
-    out = fused_moe_fp8(x.to(dev), w1q.to(dev), w1s.to(dev), w2q.to(dev), w2s.to(dev),
-                        tw.to(dev), ids.to(dev), k)
     ref = ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids)
+    d = [t.to(dev) for t in (x, w1q, w1s, w2q, w2s, tw, ids)]
+    # default choice of tile height: 128-row kernel for row-major weights, 64-row for shuffled
+    out = fm.fused_moe_fp8(*d, k)
     assert out.shape == (T, H) and out.dtype == dtype
     _check(out.cpu(), ref)
-    # operand-order weight storage: same bytes re-arranged, so the result is bit-identical
-    out2 = fused_moe_fp8(x.to(dev), shuffle_moe_weight_fp8(w1q.to(dev)), w1s.to(dev),
-                         shuffle_moe_weight_fp8(w2q.to(dev)), w2s.to(dev), tw.to(dev), ids.to(dev),
-                         k, weights_shuffled=True)
-    assert torch.equal(out2, out)
+    sh = fm.shuffle_moe_weight_fp8
+    for block in (64, 128):                      # both kernels, both weight layouts
+        monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+        plain = fm.fused_moe_fp8(*d, k)
+        _check(plain.cpu(), ref)
+        # operand-order weight storage: same bytes re-arranged, so the result is bit-identical
+        shuf = fm.fused_moe_fp8(d[0], sh(d[1]), d[2], sh(d[3]), d[4], d[5], d[6], k,
+                                weights_shuffled=True)
+        assert torch.equal(shuf, plain)
 
 
 def test_weight_shuffle_layout(dev):
