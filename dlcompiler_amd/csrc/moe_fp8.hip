@@ -487,7 +487,7 @@ __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const Mo
 // Weights may be row-major (8 lanes fetch one row's 128-byte line) or operand-order.
 // ---------------------------------------------------------------------------------------
 template <bool GATED, int DT, int QT>
-__global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmParams p) {
+__device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const int logical) {
   constexpr int BM = 128, BN = 256, MT = 4;
   constexpr int kWSlot = BN * 128;  // bytes of one weight ring slot
   constexpr int kXSlot = BM * 128;  // bytes of one activation ring slot
@@ -499,9 +499,6 @@ __global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmPara
   __shared__ float red_lds[4][BM];
   __shared__ int32_t sid_lds[BM];
 
-  const int per_xcd = gridDim.x >> 3;
-  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (logical >= p.grid_real) return;
   const int mb = logical % p.num_mblocks;
   const int nt = logical / p.num_mblocks;
   const int e_global = p.expert_ids[mb];
@@ -866,6 +863,18 @@ __global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmPara
   }
 }
 
+// Same tile walk as moe_gemm_fp8_kernel (XCD x owns a contiguous range of the logical order).
+template <bool GATED, int DT, int QT>
+__global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmParams p) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+  const int per_xcd = (p.grid_real + 7) >> 3;
+  for (int i = slot; i < per_xcd; i += slots) {
+    const int logical = xcd * per_xcd + i;
+    if (logical < p.grid_real) moe_gemm_wide_tile<GATED, DT, QT>(p, logical);
+    __syncthreads();  // the tile's LDS is reused by the next one
+  }
+}
+
 // out[t, n] = sum_j in[t * topk + j, n], fp32 accumulation in slot order, one rounding
 template <int DT>
 __global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restrict__ in,
@@ -955,8 +964,9 @@ int launch_moe_gemm(const MoeGemmParams& p, int dtype, int block_m, hipStream_t 
   const uint32_t pgrid = (GATED || grid < resident) ? grid : resident;
 #define DLB_LAUNCH_GEMM(DT_) \
   hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, 64, QT>), dim3(pgrid), dim3(256), 0, s, p)
+  const uint32_t wgrid = grid < resident / 2 ? grid : resident / 2;  // one 8-wave workgroup per CU
 #define DLB_LAUNCH_WIDE(DT_) \
-  hipLaunchKernelGGL((moe_gemm_wide_kernel<GATED, DT_, QT>), dim3(grid), dim3(512), 0, s, p)
+  hipLaunchKernelGGL((moe_gemm_wide_kernel<GATED, DT_, QT>), dim3(wgrid), dim3(512), 0, s, p)
   if (dtype == DLB_DTYPE_BF16) {
     if (block_m == 128) DLB_LAUNCH_WIDE(DLB_DTYPE_BF16);
     else DLB_LAUNCH_GEMM(DLB_DTYPE_BF16);
