@@ -727,7 +727,6 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
         read_x(x_cur, kc, 3, xq[1], asq[1]);
       }
       if (kc + 2 < KC) issue_x(kc + 2, x_tgt);
-      if (kc + 3 < KC) issue_w(kc + 3, w_cur);
       read_w(w_nxt, bn);
       if (QT == 0) {
         wsn[0] = ws_row0[(kc + 1) & (kSC - 1)];
@@ -739,6 +738,9 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     __builtin_amdgcn_sched_barrier(0);
     step(bc, 2, 0);
     __builtin_amdgcn_sched_barrier(0);
+    // the weights of chunk kc + 3 (least urgent) go out a step after the activations, which
+    // spreads the workgroup's requests; still issued after X(kc + 2), as the waits assume
+    if (kc + 3 < KC) issue_w(kc + 3, w_cur);
     if (more) read_x(x_nxt, kc + 1, 0, xq[0], asq[0]);
     __builtin_amdgcn_sched_barrier(0);
     step(bc, 3, 1);
