@@ -4,7 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
 Runs the five BASELINE.json configurations (fused silu_and_mul, MoE gating + alignment,
-varlen causal prefill attention, paged decode attention, fp8 fused-MoE MLP) on synthetic,
+varlen causal prefill attention, paged decode attention, fp8 fused-MoE MLP) and four neighbouring
+decoder-layer operators (add + RMSNorm, rotary embedding, KV-cache fill, paged prefill) on synthetic,
 seeded inputs that are resident in HBM before the timed region, and prints ONE JSON line.
 A "step" is one call of an operator's public entry point on one batch.  The top-level
 `metric`/`value`/`roofline`/`cpu_baseline` describe the primary workload (--workload, default
@@ -383,12 +384,186 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
     return res
 
 
+def _hbm_result(metric, workload, bytes_, ms, ms_kernel, kernel, dtype="bf16"):
+    return {
+        "metric": metric, "unit": "GB/s", "value": bytes_ / ms / 1e6, "ms_per_step": ms,
+        "dtype": dtype, "config": {"workload": workload, "algorithmic_bytes": bytes_},
+        "roofline": {"kernel": kernel, "bound": "hbm", "achieved": bytes_ / ms_kernel / 1e6,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": bytes_ / ms_kernel / 1e6 / PEAK_HBM_GBS, "traffic": None},
+    }
+
+
+def wl_add_rms_norm(dev, steps, warmup, cpu):
+    """Decoder-layer neighbour: residual add + RMSNorm, [16384, 4096] bf16 (read x, residual;
+    write out, new residual; the weight row is noise)."""
+    from dlcompiler_amd.kernels.rms_norm import rms_norm
+
+    M, N, nbuf = 16384, 4096, 3
+    g = _gen(6)
+    xs = [torch.randn((M, N), generator=g).bfloat16().to(dev) for _ in range(nbuf)]
+    rs = [torch.randn((M, N), generator=g).bfloat16().to(dev) for _ in range(nbuf)]
+    w = torch.randn((N,), generator=g).bfloat16().to(dev)
+    outs = [torch.empty_like(xs[0]) for _ in range(nbuf)]
+    ors = [torch.empty_like(xs[0]) for _ in range(nbuf)]
+    bytes_ = 4 * M * N * 2 + N * 2
+    ms, msk = _time_steps(lambda i: rms_norm(xs[i % nbuf], w, 1e-6, residual=rs[i % nbuf],
+                                             out=outs[i % nbuf], out_residual=ors[i % nbuf]),
+                          steps, warmup)
+    res = _hbm_result("add_rms_norm HBM GB/s", "rms_norm with residual, bf16 [16384, 4096] seed 6",
+                      bytes_, ms, msk, "rms_norm_kernel<add>")
+    if cpu:
+        from oracle import decoder_ops as od
+
+        x, r = xs[0][:2048].cpu(), rs[0][:2048].cpu()
+        t0 = time.perf_counter()
+        od.rms_norm(x, w.cpu(), 1e-6, residual=r)
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": bytes_ * 2048 / M / dt / 1e9, "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"2048 of {M} rows, 1 rep"}
+    return res
+
+
+def wl_rotary(dev, steps, warmup, cpu):
+    """Decoder-layer neighbour: rotary embedding of q [16384, 32, 128] and k [16384, 8, 128]."""
+    from dlcompiler_amd.kernels.apply_rotary_pos_emb import apply_rotary_pos_emb
+
+    T, HQ, HK, D, nbuf = 16384, 32, 8, 128, 3
+    g = _gen(7)
+    qs = [torch.randn((T, HQ, D), generator=g).bfloat16().to(dev) for _ in range(nbuf)]
+    ks = [torch.randn((T, HK, D), generator=g).bfloat16().to(dev) for _ in range(nbuf)]
+    ang = torch.rand((T, D // 2), generator=g) * 6.28
+    cos = torch.cat([ang.cos(), ang.cos()], -1).bfloat16().to(dev)
+    sin = torch.cat([ang.sin(), ang.sin()], -1).bfloat16().to(dev)
+    qo = [torch.empty_like(qs[0]) for _ in range(nbuf)]
+    ko = [torch.empty_like(ks[0]) for _ in range(nbuf)]
+    bytes_ = 2 * T * (HQ + HK) * D * 2 + 2 * T * D * 2
+    ms, msk = _time_steps(lambda i: apply_rotary_pos_emb(qs[i % nbuf], ks[i % nbuf], cos, sin,
+                                                         qo[i % nbuf], ko[i % nbuf]), steps, warmup)
+    res = _hbm_result("apply_rotary_pos_emb HBM GB/s",
+                      "apply_rotary_pos_emb bf16 q [16384, 32, 128], k [16384, 8, 128] seed 7",
+                      bytes_, ms, msk, "rotary_kernel")
+    if cpu:
+        from oracle import decoder_ops as od
+
+        n = 2048
+        t0 = time.perf_counter()
+        od.apply_rotary_pos_emb(qs[0][:n].cpu(), ks[0][:n].cpu(), cos[:n, None].cpu(), sin[:n, None].cpu())
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": bytes_ * n / T / dt / 1e9, "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{n} of {T} tokens, 1 rep"}
+    return res
+
+
+def wl_fill_kv_cache(dev, steps, warmup, cpu):
+    """The step before attention: scatter the new K/V rows of a prefill batch (config-3
+    lengths) into 64-token pages, 8 KV heads, d128."""
+    from dlcompiler_amd.kernels.fill_kv_cache import fill_kv_cache
+
+    g = _gen(2)
+    B, HKV, D, PAGE = 8, 8, 128, 64
+    lens = torch.randint(512, 4097, (B,), generator=g)
+    T = int(lens.sum())
+    blocks = (lens + PAGE - 1) // PAGE
+    num_pages = int(blocks.sum())
+    perm = torch.randperm(num_pages, generator=g).to(torch.int32)
+    table = torch.zeros((B, int(blocks.max())), dtype=torch.int32)
+    at = 0
+    for b in range(B):
+        table[b, :blocks[b]] = perm[at:at + blocks[b]]
+        at += int(blocks[b])
+    nbuf = 2
+    k = [torch.randn((T, HKV, D), generator=g).bfloat16().to(dev) for _ in range(nbuf)]
+    v = [torch.randn((T, HKV, D), generator=g).bfloat16().to(dev) for _ in range(nbuf)]
+    kc = [torch.zeros((num_pages, PAGE, HKV, D), dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+    vc = [torch.zeros((num_pages, PAGE, HKV, D), dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+    start = (torch.cumsum(lens, 0) - lens).to(torch.int32).to(dev)
+    lens_d, table_d = lens.to(torch.int32).to(dev), table.to(dev)
+    bytes_ = 4 * T * HKV * D * 2
+    ms, msk = _time_steps(lambda i: fill_kv_cache(k[i % nbuf], v[i % nbuf], kc[i % nbuf], vc[i % nbuf],
+                                                  start, lens_d, lens_d, int(lens.max()), table_d),
+                          steps, warmup)
+    res = _hbm_result("fill_kv_cache HBM GB/s",
+                      f"fill_kv_cache bf16, 8 seqs U[512,4096] seed 2 ({T} tokens), 8 kv heads, d128, 64-token pages",
+                      bytes_, ms, msk, "fill_kv_cache_kernel")
+    if cpu:
+        from oracle import decoder_ops as od
+
+        t0 = time.perf_counter()
+        od.fill_kv_cache(k[0][:int(lens[0])].cpu(), v[0][:int(lens[0])].cpu(), kc[0].cpu(), vc[0].cpu(),
+                         [int(lens[0])], [0], table[:1])
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": bytes_ * int(lens[0]) / T / dt / 1e9, "unit": "GB/s",
+                               "cores": 1, "kind": "port",
+                               "sample": f"first sequence ({int(lens[0])} tokens), 1 rep (includes a copy of the cache)"}
+    return res
+
+
+def wl_paged_prefill(dev, steps, warmup, cpu):
+    """Chunked prefill: 8 sequences, 512 new tokens each after a history U[512, 4096] already in
+    the paged cache (paged_attention_fwd, non-decoding branch)."""
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+
+    g = _gen(8)
+    B, HQ, HKV, D, PAGE, QL = 8, 32, 8, 128, 64, 512
+    hist = torch.randint(512, 4097, (B,), generator=g)
+    kvl = hist + QL
+    blocks = (kvl + PAGE - 1) // PAGE
+    num_pages = int(blocks.sum())
+    perm = torch.randperm(num_pages, generator=g).to(torch.int32)
+    table = torch.zeros((B, int(blocks.max())), dtype=torch.int32)
+    at = 0
+    for b in range(B):
+        table[b, :blocks[b]] = perm[at:at + blocks[b]]
+        at += int(blocks[b])
+    kc = torch.randn((num_pages, PAGE, HKV, D), generator=g).bfloat16().to(dev)
+    vc = torch.randn((num_pages, PAGE, HKV, D), generator=g).bfloat16().to(dev)
+    q = torch.randn((B * QL, HQ, D), generator=g).bfloat16().to(dev)
+    o = torch.empty_like(q)
+    start = (torch.arange(B) * QL).to(torch.int32).to(dev)
+    ql = torch.full((B,), QL, dtype=torch.int32, device=dev)
+    kvl_d, table_d = kvl.to(torch.int32).to(dev), table.to(dev)
+    pairs = sum(QL * int(h) + QL * (QL + 1) // 2 for h in hist)
+    flops = 4 * D * HQ * pairs
+    ms, msk = _time_steps(lambda i: paged_attention_fwd(q, kc, vc, o, table_d, start, ql, kvl_d, QL),
+                          steps, warmup)
+    res = {
+        "metric": "paged prefill attention TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
+        "ms_per_step": ms, "dtype": "bf16",
+        "config": {"workload": "paged_attention_fwd prefill, 8 seqs x 512 new tokens after history "
+                               "U[512,4096] seed 8, 64-token pages, 32q/8kv heads, d128, bf16",
+                   "algorithmic_flops": flops},
+        "roofline": {"kernel": "prefill_attn_kernel<paged>", "bound": "mfma",
+                     "achieved": flops / msk / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / msk / 1e9 / PEAK_BF16_TFLOPS, "traffic": None},
+    }
+    if cpu:
+        from oracle import attention as oa
+
+        t0 = time.perf_counter()
+        oa.paged_prefill(q[:QL].cpu(), kc.cpu(), vc.cpu(), table[:1], torch.tensor([0]),
+                         torch.tensor([QL]), kvl[:1])
+        dt = time.perf_counter() - t0
+        f1 = 4 * D * HQ * (QL * int(hist[0]) + QL * (QL + 1) // 2)
+        res["cpu_baseline"] = {"value": f1 / dt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "first sequence, 1 rep"}
+    return res
+
+
 WORKLOADS = {
     "silu_and_mul": wl_silu,
     "moe_gating": wl_gating,
     "prefill_attention": wl_prefill,
     "paged_decode": wl_decode,
     "moe_fp8": wl_moe_fp8,
+    # the neighbours of the five configurations in a decoder layer
+    "add_rms_norm": wl_add_rms_norm,
+    "apply_rotary_pos_emb": wl_rotary,
+    "fill_kv_cache": wl_fill_kv_cache,
+    "paged_prefill": wl_paged_prefill,
 }
 PRIMARY = "moe_fp8"
 

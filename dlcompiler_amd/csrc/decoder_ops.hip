@@ -14,7 +14,7 @@ namespace {
 
 // ---------------------------------------------------------------------------------------
 // fill_kv_cache: token t of sequence b (its i-th new token) goes to cache position
-// history_b + i, i.e. page block_offsets[b][pos / page], slot pos % page.  One workgroup per
+// history_b + i, i.e. page block_offsets[b][pos / page], slot pos % page.  One wavefront per
 // new token; rows are copied as bytes in 16-byte chunks (H * D * elem bytes per token).
 // ---------------------------------------------------------------------------------------
 struct FillParams {
@@ -29,50 +29,61 @@ struct FillParams {
   int64_t ks_tok, ks_head, vs_tok, vs_head;              // bytes
   int64_t kc_page, kc_slot, kc_head, vc_page, vc_slot, vc_head;  // bytes
   int64_t bt_stride;
+  int64_t num_tokens;
   int batch, heads, page, max_blocks;
   int k_row_bytes, v_row_bytes;  // head_dim * elem, head_dim_v * elem
   int vec;                       // 1: 16-byte chunks, 0: single bytes
 };
 
-__global__ __launch_bounds__(256) void fill_kv_cache_kernel(const FillParams p) {
-  __shared__ int seq_s;
-  const int t = blockIdx.x;
-  if (threadIdx.x == 0) seq_s = -1;
-  __syncthreads();
-  for (int b = threadIdx.x; b < p.batch; b += 256) {
-    const int s0 = p.q_start[b], n = p.q_len[b];
-    if (t >= s0 && t < s0 + n) seq_s = b;  // sequences do not overlap: at most one writer
+constexpr int kFillTokens = 4;  // tokens (= wavefronts) per workgroup
+
+// One wavefront per new token: it finds the sequence that owns the token with a ballot over
+// the batch, then streams the token's K and V rows into the page slot (no barriers).
+__global__ __launch_bounds__(64 * kFillTokens) void fill_kv_cache_kernel(const FillParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * kFillTokens + (threadIdx.x >> 6);
+  if (t >= p.num_tokens) return;
+  int b = -1;
+  for (int b0 = 0; b0 < p.batch && b < 0; b0 += 64) {
+    const int bb = b0 + lane;
+    bool hit = false;
+    if (bb < p.batch) {
+      const int s0 = p.q_start[bb], n = p.q_len[bb];
+      hit = t >= s0 && t < (int64_t)s0 + n;
+    }
+    const uint64_t m = __ballot(hit);
+    if (m) b = b0 + __builtin_ctzll(m);  // sequences do not overlap: at most one owner
   }
-  __syncthreads();
-  const int b = seq_s;
   if (b < 0) return;
-  const int i = t - p.q_start[b];
+  const int i = (int)(t - p.q_start[b]);
   const int pos = p.kv_len[b] - p.q_len[b] + i;
   const int pi = pos / p.page;
   if (pos < 0 || pi >= p.max_blocks) return;
   const int64_t pg = p.block_table[(int64_t)b * p.bt_stride + pi];
   const int slot = pos - pi * p.page;
 
-  const unsigned char* ksrc = p.ks + (int64_t)t * p.ks_tok;
-  const unsigned char* vsrc = p.vs + (int64_t)t * p.vs_tok;
+  const unsigned char* ksrc = p.ks + t * p.ks_tok;
+  const unsigned char* vsrc = p.vs + t * p.vs_tok;
   unsigned char* kdst = p.kc + pg * p.kc_page + (int64_t)slot * p.kc_slot;
   unsigned char* vdst = p.vc + pg * p.vc_page + (int64_t)slot * p.vc_slot;
   if (p.vec) {
     const int kc_per_head = p.k_row_bytes >> 4, vc_per_head = p.v_row_bytes >> 4;
-    for (int u = threadIdx.x; u < p.heads * kc_per_head; u += 256) {
+    for (int u = lane; u < p.heads * kc_per_head; u += 64) {
       const int h = u / kc_per_head, c = u - h * kc_per_head;
-      *(u32x4*)(kdst + h * p.kc_head + c * 16) = *(const u32x4*)(ksrc + h * p.ks_head + c * 16);
+      __builtin_nontemporal_store(__builtin_nontemporal_load((const u32x4*)(ksrc + h * p.ks_head + c * 16)),
+                                  (u32x4*)(kdst + h * p.kc_head + c * 16));
     }
-    for (int u = threadIdx.x; u < p.heads * vc_per_head; u += 256) {
+    for (int u = lane; u < p.heads * vc_per_head; u += 64) {
       const int h = u / vc_per_head, c = u - h * vc_per_head;
-      *(u32x4*)(vdst + h * p.vc_head + c * 16) = *(const u32x4*)(vsrc + h * p.vs_head + c * 16);
+      __builtin_nontemporal_store(__builtin_nontemporal_load((const u32x4*)(vsrc + h * p.vs_head + c * 16)),
+                                  (u32x4*)(vdst + h * p.vc_head + c * 16));
     }
   } else {
-    for (int u = threadIdx.x; u < p.heads * p.k_row_bytes; u += 256) {
+    for (int u = lane; u < p.heads * p.k_row_bytes; u += 64) {
       const int h = u / p.k_row_bytes, c = u - h * p.k_row_bytes;
       kdst[h * p.kc_head + c] = ksrc[h * p.ks_head + c];
     }
-    for (int u = threadIdx.x; u < p.heads * p.v_row_bytes; u += 256) {
+    for (int u = lane; u < p.heads * p.v_row_bytes; u += 64) {
       const int h = u / p.v_row_bytes, c = u - h * p.v_row_bytes;
       vdst[h * p.vc_head + c] = vsrc[h * p.vs_head + c];
     }
@@ -245,6 +256,7 @@ extern "C" int dlb_fill_kv_cache(const void* k_states, const void* v_states, voi
   p.vc_head = vc_stride_head * es;
   p.bt_stride = bt_stride;
   p.batch = batch;
+  p.num_tokens = num_tokens;
   p.heads = heads;
   p.page = page;
   p.max_blocks = max_blocks;
@@ -254,8 +266,8 @@ extern "C" int dlb_fill_kv_cache(const void* k_states, const void* v_states, voi
           mult16(p.k_row_bytes) && mult16(p.v_row_bytes) && mult16(p.ks_tok) && mult16(p.ks_head) &&
           mult16(p.vs_tok) && mult16(p.vs_head) && mult16(p.kc_page) && mult16(p.kc_slot) &&
           mult16(p.kc_head) && mult16(p.vc_page) && mult16(p.vc_slot) && mult16(p.vc_head);
-  hipLaunchKernelGGL(fill_kv_cache_kernel, dim3((uint32_t)num_tokens), dim3(256), 0,
-                     (hipStream_t)stream, p);
+  hipLaunchKernelGGL(fill_kv_cache_kernel, dim3((uint32_t)ceil_div(num_tokens, kFillTokens)),
+                     dim3(64 * kFillTokens), 0, (hipStream_t)stream, p);
   return launch_status();
 }
 
