@@ -48,34 +48,46 @@ __device__ __forceinline__ unsigned int pack4_fp8(float a, float b, float c, flo
 // ---------------------------------------------------------------------------------------
 // per-token-group quantisation: one DPP row (16 lanes x 8 elements) per 128-element group
 // ---------------------------------------------------------------------------------------
+constexpr int kQuantUnroll = 4;  // groups per DPP row and workgroup pass (loads issued together)
+
 template <int DT>
 __global__ __launch_bounds__(256) void quant_fp8_group128_kernel(
     const unsigned short* __restrict__ x, unsigned char* __restrict__ xq, float* __restrict__ xs,
     int64_t total_groups, int groups_per_row, int64_t ldx, int64_t ldq, int64_t lds) {
   const int lane16 = threadIdx.x & 15;
-  const int64_t gidx = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const bool live = gidx < total_groups;
-  const int64_t row = live ? gidx / groups_per_row : 0;
-  const int gc = live ? (int)(gidx - row * groups_per_row) : 0;
-  u32x4 raw = u32x4{0u, 0u, 0u, 0u};
-  if (live) raw = *(const u32x4*)(x + row * ldx + gc * 128 + lane16 * 8);
-  float v[8];
+  int64_t row[kQuantUnroll];
+  int gc[kQuantUnroll];
+  bool live[kQuantUnroll];
+  u32x4 raw[kQuantUnroll];
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    v[2 * w] = Elem<DT>::lo(raw[w]);
-    v[2 * w + 1] = Elem<DT>::hi(raw[w]);
+  for (int u = 0; u < kQuantUnroll; ++u) {
+    const int64_t gidx = ((int64_t)blockIdx.x * kQuantUnroll + u) * 16 + (threadIdx.x >> 4);
+    live[u] = gidx < total_groups;
+    row[u] = live[u] ? gidx / groups_per_row : 0;
+    gc[u] = live[u] ? (int)(gidx - row[u] * groups_per_row) : 0;
+    raw[u] = u32x4{0u, 0u, 0u, 0u};
+    if (live[u]) raw[u] = __builtin_nontemporal_load((const u32x4*)(x + row[u] * ldx + gc[u] * 128 + lane16 * 8));
   }
-  float amax = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-  amax = row16_max(amax);
-  const float scale = fmaxf(amax, kQuantEps) / kFp8Max;
-  if (live) {
-    u32x2 q;
-    q[0] = pack4_fp8(v[0] / scale, v[1] / scale, v[2] / scale, v[3] / scale);
-    q[1] = pack4_fp8(v[4] / scale, v[5] / scale, v[6] / scale, v[7] / scale);
-    *(u32x2*)(xq + row * ldq + gc * 128 + lane16 * 8) = q;
-    if (lane16 == 0) xs[row * lds + gc] = scale;
+  for (int u = 0; u < kQuantUnroll; ++u) {
+    float v[8];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      v[2 * w] = Elem<DT>::lo(raw[u][w]);
+      v[2 * w + 1] = Elem<DT>::hi(raw[u][w]);
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = row16_max(amax);
+    const float scale = fmaxf(amax, kQuantEps) / kFp8Max;
+    if (live[u]) {
+      u32x2 q;
+      q[0] = pack4_fp8(v[0] / scale, v[1] / scale, v[2] / scale, v[3] / scale);
+      q[1] = pack4_fp8(v[4] / scale, v[5] / scale, v[6] / scale, v[7] / scale);
+      *(u32x2*)(xq + row[u] * ldq + gc[u] * 128 + lane16 * 8) = q;
+      if (lane16 == 0) xs[row[u] * lds + gc[u]] = scale;
+    }
   }
 }
 
@@ -919,7 +931,7 @@ extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs,
     return DLB_ERR_UNSUPPORTED;
   const int gpr = K / 128;
   const int64_t total = M * gpr;
-  const dim3 grid((uint32_t)ceil_div(total, 16));
+  const dim3 grid((uint32_t)ceil_div(total, 16 * kQuantUnroll));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DLB_DTYPE_BF16)
     hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_BF16>, grid, dim3(256), 0, s,
