@@ -107,6 +107,37 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// wave-uniform LDS byte address of a pointer into __shared__ memory, in a scalar register
+__device__ __forceinline__ unsigned int lds_addr(const void* p) {
+  typedef const __attribute__((address_space(3))) void* lds_ptr_t;
+  return (unsigned int)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(lds_ptr_t)p);
+}
+// Direct global -> LDS copy of 16 bytes per lane: lane l's bytes land at lds_base + 16 * l
+// (lds_base: wave-uniform LDS byte address).  Issued through inline assembly rather than
+// __builtin_amdgcn_global_load_lds because the compiler's wait-count pass models the builtin as
+// a FLAT access that may complete out of order with LDS reads: while one is in flight every
+// LDS wait it inserts becomes lgkmcnt(0), which serialises a pipelined ds_read -> MFMA stream.
+// The copy is counted by vmcnt like any other vector load (loads return in order); the compiler
+// does not see it, so the caller waits for it explicitly (s_waitcnt vmcnt) before the barrier
+// that publishes the data.  Waits the compiler inserts for its own loads stay correct: an
+// unseen load that is older completes first, one that is younger only makes the wait longer.
+__device__ __forceinline__ void dma16_global_to_lds(const void* gsrc, unsigned int lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_base)
+               : "memory");
+}
+
+// ds_read_b64_tr_b16: every lane passes the address of four consecutive 16-bit elements; in
+// each group of 16 lanes the 16 x 4 elements form a 4-row x 16-column block (row j = lanes
+// 4j .. 4j+3 of the group, four columns each) and lane l of the group receives column l,
+// rows 0..3, lowest row in the low half of the first register.
+__device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
+  typedef __attribute__((ext_vector_type(4))) short s16x4;
+  typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p));
+}
+
 __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) {
   return (a + b - 1) / b;
 }

@@ -5,14 +5,16 @@
 // (sequence, query head, query tile) stream the causal prefix of K/V, QK^T in fp32, online
 // softmax, P rounded to the input dtype before P.V -- re-tiled for CDNA4:
 //   * a workgroup of 4 wavefronts owns 128 query rows (32 per wave) and walks 64-key K/V tiles
-//     that are double-buffered in LDS (global -> registers -> LDS, one barrier per tile);
+//     that are double-buffered in LDS (copied global -> LDS directly, one barrier per tile);
 //   * S^T = K.Q^T and O^T = V^T.P^T on 32x32x16 MFMA.  Working on the transposes puts a query
 //     in a lane *column*: the row max/sum are register reductions plus one exchange between
-//     the two lane halves, the rescale is a per-lane scalar, and with the key order inside a
-//     32-key tile permuted at V-staging time the softmax output registers are already the B
-//     operand of the second product (P never crosses lanes);
-//   * V is transposed on its way into LDS (4 keys x 8 dims per lane, v_perm + ds_write_b64),
-//     K is stored row-major; both are read back as 128-bit MFMA operands;
+//     the two lane halves, the rescale is a per-lane scalar, and the softmax output registers
+//     are already the B operand of the second product (P never crosses lanes): the V^T
+//     operand is simply fetched in the key order those registers have;
+//   * K and V both sit row-major in LDS.  K fragments are 128-bit reads; V^T fragments come
+//     from ds_read_b64_tr_b16, which hands lane l of a 16-lane group column l of a 4-row x
+//     16-column block (rows supplied by lanes 4j .. 4j+3), i.e. the transpose happens in the
+//     LDS read and V never passes through registers on its way in;
 //   * the exponent runs in base 2 with the softmax scale folded into one FMA;
 //   * fully masked tiles are skipped per wave and only diagonal tiles pay for the mask; the
 //     heaviest query tiles are launched first.
@@ -83,8 +85,7 @@ template <int D>
 struct Smem {
   static constexpr int kRowBytes = D * 2;           // K: [64][D], 16-byte chunks XOR-swizzled
   static constexpr int kBytes = kTileN * kRowBytes;
-  static constexpr int vRowBytes = kTileN * 2;       // V^T: [D][64], 16-byte units XOR-swizzled
-  static constexpr int vBytes = D * vRowBytes;
+  static constexpr int vBytes = kBytes;              // V: [64][D], 16-byte chunks XOR-swizzled
   static constexpr int stage = kBytes + vBytes;
 };
 
@@ -95,8 +96,6 @@ template <int DT, int D, bool PAGED>
 __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int KS = D / 16;  // MFMA k-steps over the head dim for S^T
   constexpr int MT = D / 32;  // 32-row tiles of O^T
-  constexpr int VUNITS = (kTileN / 4) * (D / 8);    // (4 keys x 8 dims) units per tile
-  constexpr int VLD = (VUNITS + kThreads - 1) / kThreads;
   constexpr int DG = D / 8;
   using SM = Smem<D>;
 
@@ -151,87 +150,69 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   const int qpos = hist + qrow;                          // context position of this lane's query
   const int wave_last_pos = hist + q0 + 32 * wave + 31;
 
-  // ---- global -> register staging of one K/V tile.  Per-thread base pointers are formed
-  // once; a tile adds a workgroup-uniform offset.  CLAMP (tiles that may run past the
-  // sequence) redirects rows >= L to row L-1 so nothing outside the sequence is read.
-  // K goes global -> LDS directly (global_load_lds_dwordx4: lane l's 16 bytes land at
-  // base + 16*l, so one wave instruction fills 1 KB = 1024 / (2*D) rows).  Rows are stored
-  // unpadded; bank conflicts are avoided by letting lane (row r, position c) fetch global
-  // chunk c ^ (r & 15): a reader that wants chunk c of row r reads position c ^ (r & 15).
+  // ---- global -> LDS staging of one K/V tile.  Per-thread base pointers are formed once; a
+  // tile adds a workgroup-uniform offset.  CLAMP (tiles that may run past the sequence)
+  // redirects rows >= kv_total to the last row so nothing outside the sequence is read.
+  // Both operands go global -> LDS directly (global_load_lds_dwordx4: lane l's 16 bytes land
+  // at base + 16*l, so one wave instruction fills 1 KB = 1024 / (2*D) rows).  Rows are stored
+  // unpadded; bank conflicts are avoided by permuting which 16-byte chunk of its row a lane
+  // fetches: position c of row r holds chunk c ^ swz(r), so a reader that wants chunk c of
+  // row r reads position c ^ swz(r).  K: swz(r) = r mod DG (128-bit fragment reads, one row
+  // per lane).  V: swz(r) spreads the 4 (or 8) rows that one transposing read touches over
+  // all banks.
   constexpr int KRPI = 1024 / (2 * D);            // rows per wave instruction
-  constexpr int KINS = kTileN / KRPI / 4;         // instructions per wave and tile
+  constexpr int KINS = kTileN / KRPI / 4;         // instructions per wave, tile and operand
   const int k_lrow = lane / DG;                   // row inside an instruction
   const int k_pos = lane % DG;                    // 16-byte position inside the row
   const unsigned char* kbytes = (const unsigned char*)kb;
-  const unsigned char* vbytes = (const unsigned char*)vb + 16 * (tid % DG);
+  const unsigned char* vbytes = (const unsigned char*)vb;
   const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
   const int32_t* bt = PAGED ? p.block_table + (int64_t)seq * p.bt_stride : nullptr;
-  // byte address of key row `key` of this sequence (page lookup for the paged layout)
-  auto k_row = [&](int key) -> const unsigned char* {
-    if (PAGED) {
-      const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
-      return kbytes + ((int64_t)bt[pi] * p.k_sp + (int64_t)(key - pi * p.page) * p.k_st) * 2;
-    }
-    return kbytes + (tok0 + key) * k_row_bytes;
+  // V chunk swizzle of row r (depends on r mod 8 only)
+  auto v_swz = [](int r) -> int {
+    return D == 128 ? (((r & 3) << 2) | (((r >> 2) & 1) << 1))
+                    : ((((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1));
   };
-  auto v_row = [&](int key) -> const unsigned char* {
-    if (PAGED) {
-      const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
-      return vbytes + ((int64_t)bt[pi] * p.v_sp + (int64_t)(key - pi * p.page) * p.v_st) * 2;
+  // paged layout: the page ids of the rows this lane copies are fetched one tile ahead of the
+  // copy that needs them, so the block-table latency never sits in front of a tile's copies
+  int pg_next[KINS];
+  auto fetch_pages = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < KINS; ++i) {
+      const int key = min(t0 + (4 * i + wave) * KRPI + k_lrow, kv_total - 1);
+      pg_next[i] = bt[p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page)];
     }
-    return vbytes + (tok0 + key) * v_row_bytes;
   };
-  const bool v_active = (VUNITS >= kThreads) || (tid < VUNITS);
-  u32x4 vreg[4];
-  static_assert(VLD == 1, "one (4 keys x 8 dims) V unit per thread");
   auto load_tile = [&](auto clamp_tag, int t0, int buf) {
     constexpr bool CLAMP = decltype(clamp_tag)::value;
     unsigned char* ks = smem + buf * SM::stage;
+    unsigned char* vs = ks + SM::kBytes;
+    const unsigned char* ksrc[KINS];
+    const unsigned char* vsrc[KINS];
 #pragma unroll
     for (int i = 0; i < KINS; ++i) {
-      const int q = 4 * i + wave;                 // which 1 KB slice of the tile
-      const int r = q * KRPI + k_lrow;            // key row inside the tile
+      const int r = (4 * i + wave) * KRPI + k_lrow;  // key row inside the tile
       int key = t0 + r;
       if (CLAMP) key = min(key, kv_total - 1);
-      const unsigned char* src = k_row(key) + ((k_pos ^ (r & (DG - 1))) << 4);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(ks + q * 1024),
-                                       16, 0, 0);
-    }
-    if (v_active) {
-      // the 4 keys of a unit share a page (page % 4 == 0)
-      const int key0 = t0 + 4 * (tid / DG);
-      const unsigned char* v0 = v_row(CLAMP ? min(key0, kv_total - 1) : key0);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int rr = CLAMP ? max(min(r, kv_total - 1 - key0), 0) : r;
-        vreg[r] = *(const u32x4*)(v0 + rr * v_row_bytes);
+      if (PAGED) {
+        const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
+        const int64_t slot = key - pi * p.page;
+        ksrc[i] = kbytes + ((int64_t)pg_next[i] * p.k_sp + slot * p.k_st) * 2;
+        vsrc[i] = vbytes + ((int64_t)pg_next[i] * p.v_sp + slot * p.v_st) * 2;
+      } else {
+        ksrc[i] = kbytes + (tok0 + key) * k_row_bytes;
+        vsrc[i] = vbytes + (tok0 + key) * v_row_bytes;
       }
+      ksrc[i] += (k_pos ^ (r & (DG - 1))) << 4;
+      vsrc[i] += (k_pos ^ v_swz(r)) << 4;
     }
-  };
-  // LDS addresses of this thread's staging slots (tile-independent)
-  const int st_kg = tid / DG, st_dg = tid % DG;
-  // key = 32*nt + 16*st + 8*a + 4*h + r  ->  position 32*nt + 16*st + 8*h + 4*a + r
-  const int st_unit = ((st_kg >> 2) << 1) | (st_kg & 1);  // 16-byte unit 4*nt + 2*st + h
-  const int st_half = (st_kg >> 1) & 1;                   // 8-byte half a
-  auto store_tile = [&](int buf) {
-    unsigned char* vs = smem + buf * SM::stage + SM::kBytes;
-    if (v_active) {
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const unsigned int lo01 = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], 0x05040100u);
-        const unsigned int lo23 = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], 0x05040100u);
-        const unsigned int hi01 = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], 0x07060302u);
-        const unsigned int hi23 = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], 0x07060302u);
-        const int d0 = 8 * st_dg + 2 * w;
-        // unit swizzle (same for d0 and d0 + 1): with it the fragment reads below run at the
-        // full LDS rate and these transposing writes at half of theirs
-        const int sw = ((d0 >> 1) ^ (d0 >> 4)) & 7;
-        unsigned char* row = vs + d0 * SM::vRowBytes + ((st_unit ^ sw) << 4) + (st_half << 3);
-        *(u32x2*)(row) = u32x2{lo01, lo23};
-        *(u32x2*)(row + SM::vRowBytes) = u32x2{hi01, hi23};
-      }
+    for (int i = 0; i < KINS; ++i) {
+      const int q = 4 * i + wave;  // which 1 KB slice of the tile
+      dma16_global_to_lds(ksrc[i], lds_addr(ks + q * 1024));
+      dma16_global_to_lds(vsrc[i], lds_addr(vs + q * 1024));
     }
+    if (PAGED) fetch_pages(t0 + kTileN);
   };
 
   f32x16 o[MT];
@@ -247,6 +228,17 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   float m_run = -__builtin_inff();
   float l_run = 0.0f;  // this lane half's share of the denominator
   const float cs = p.scale_log2e;
+
+  // byte offsets of this lane's transposing V reads inside a tile, one per 32-dim block
+  int v_off[MT];
+  {
+    const int s16 = lane & 15, dhalf = (lane >> 4) & 1;
+    const int r = 4 * hh + (s16 >> 2);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      v_off[mt] = r * SM::kRowBytes +
+                  (((4 * mt + 2 * dhalf + ((s16 >> 1) & 1)) ^ v_swz(r)) << 4) + 8 * (s16 & 1);
+  }
 
   // one K/V tile against this wave's 32 queries; MASK: apply the causal mask
   auto process_tile = [&](auto mask_tag, int j) {
@@ -332,7 +324,11 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     }
     l_run += psum;
 
-    // ---- O^T += V^T . P^T ; step (nt, st) consumes registers 8*st .. 8*st+7 of s[nt]
+    // ---- O^T += V^T . P^T ; step (nt, st) consumes registers 8*st .. 8*st+7 of s[nt], which
+    // belong to keys 32*nt + 16*st + 8*a + 4*hh + r (slot e = 4*a + r).  The A operand wants,
+    // for dim d = 32*mt + col, the same 8 keys: two transposing reads (a = 0, 1), in each of
+    // which lane s of 16-lane group g supplies row 4*hh + (s >> 2) (+ the step's key base),
+    // dims 32*mt + 16*(g & 1) + 4*(s & 3) .. +3.
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
@@ -342,13 +338,12 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
         pf[1] = Mma32<DT>::pack2(s[nt][8 * st + 2], s[nt][8 * st + 3]);
         pf[2] = Mma32<DT>::pack2(s[nt][8 * st + 4], s[nt][8 * st + 5]);
         pf[3] = Mma32<DT>::pack2(s[nt][8 * st + 6], s[nt][8 * st + 7]);
-        const int unit = 4 * nt + 2 * st + hh;
+        const unsigned char* vstep = vs + (32 * nt + 16 * st) * SM::kRowBytes;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          const int d = 32 * mt + col;
-          const int sw = ((d >> 1) ^ (d >> 4)) & 7;
-          const u32x4 a = *(const u32x4*)(vs + d * SM::vRowBytes + ((unit ^ sw) << 4));
-          o[mt] = Mma32<DT>::run(a, pf, o[mt]);
+          const u32x2 lo = lds_read_tr16(vstep + v_off[mt]);
+          const u32x2 hi = lds_read_tr16(vstep + v_off[mt] + 8 * SM::kRowBytes);
+          o[mt] = Mma32<DT>::run(u32x4{lo[0], lo[1], hi[0], hi[1]}, pf, o[mt]);
         }
       }
     }
@@ -360,8 +355,8 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   // the buffer (encoding: vmcnt = 0, expcnt / lgkmcnt left at their maxima)
   auto wait_dma = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
   int j = jfirst;
+  if (PAGED) fetch_pages(j * kTileN);
   if (j < nfull) load_tile(NoClamp{}, j * kTileN, j & 1); else load_tile(Clamp{}, j * kTileN, j & 1);
-  store_tile(j & 1);
   wait_dma();
   __syncthreads();
 
@@ -369,7 +364,6 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   for (; j + 1 < nfull; ++j) {
     load_tile(NoClamp{}, (j + 1) * kTileN, (j + 1) & 1);
     process_tile(std::integral_constant<bool, false>{}, j);
-    store_tile((j + 1) & 1);
     wait_dma();
     __syncthreads();
   }
@@ -379,7 +373,6 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     if (more) load_tile(Clamp{}, (j + 1) * kTileN, (j + 1) & 1);
     if (j < nfull) process_tile(std::integral_constant<bool, false>{}, j);
     else process_tile(std::integral_constant<bool, true>{}, j);
-    if (more) store_tile((j + 1) & 1);
     wait_dma();
     __syncthreads();
   }
@@ -510,7 +503,6 @@ extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const 
   if (B == 0 || max_q_len == 0) return DLB_OK;
   if (!q || !k_cache || !v_cache || !o || !block_table || !q_start_loc || !q_len || !kv_len)
     return DLB_ERR_BAD_ARG;
-  if (page % 4 != 0) return DLB_ERR_UNSUPPORTED;  // a 4-key V unit must not straddle pages
   PrefillParams p = {};
   p.q = q;
   p.k = k_cache;

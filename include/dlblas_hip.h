@@ -153,7 +153,7 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
  *   keys >= position - window_size (:429-431,457-458); logit_softcapping > 0 replaces the
  *   scaled logits by cap * tanh(logits / cap) (:450-453).  Pass <= 0 to disable either.
  *   max_q_len >= max(q_len) sizes the grid.
- * Supported: dtype bf16/f16, D in {64, 128}, page % 4 == 0, sm_scale > 0, q/k/v strides
+ * Supported: dtype bf16/f16, D in {64, 128}, any page size >= 1, sm_scale > 0, q/k/v strides
  * multiples of 8 and bases 16-byte aligned, o strides multiples of 4 and base 8-byte aligned.
  * ---------------------------------------------------------------------------------------- */
 int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, void* o,

@@ -104,6 +104,14 @@ def test_large_chunked_prefill(dev):
     _run_case(dev, [512, 256], [3000, 1500], 8, 2, 128, 64, torch.bfloat16, seed=5)
 
 
+# pages that are neither a power of two nor a multiple of a tile: every K/V row is looked up on
+# its own, so tiles may straddle pages anywhere
+@pytest.mark.parametrize("page", [20, 24, 100])
+def test_odd_page_sizes(dev, page):
+    _run_case(dev, [70, 33, 129], [45, 0, 200], 4, 2, 128, page, torch.bfloat16, seed=page)
+    _run_case(dev, [65], [130], 2, 1, 64, page, torch.float16, seed=page + 1, window=40)
+
+
 def test_grid_larger_than_needed_and_rejects(dev):
     from dlcompiler_amd import _lib
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
