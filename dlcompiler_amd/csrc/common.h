@@ -124,7 +124,16 @@ __device__ __forceinline__ unsigned int lds_addr(const void* p) {
 __device__ __forceinline__ void dma16_global_to_lds(const void* gsrc, unsigned int lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
-               : "v"(gsrc), "s"(lds_base)
+               : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base))
+               : "memory");
+}
+
+// same copy, addressed as a wave-uniform 64-bit base (scalar registers) plus a 32-bit lane offset
+__device__ __forceinline__ void dma16_global_to_lds(const void* sbase, unsigned int voff,
+                                                    unsigned int lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane((int)lds_base))
                : "memory");
 }
 

@@ -562,24 +562,21 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   }
   const unsigned char* wbase = p.w + (int64_t)e * p.N * K;
   const int w_kc_stride = p.w_layout ? 2048 : 128;
-  typedef const __attribute__((address_space(1))) void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
   // address = uniform base (scalar registers) + 32-bit lane offset: no 64-bit vector math
+  const unsigned int w_dst0 = lds_addr(w_lds) + w * 4096, x_dst0 = lds_addr(x_lds) + w * 2048;
   auto issue_w = [&](int kc, int slot) {
     const uint32_t koff = (uint32_t)kc * (uint32_t)w_kc_stride;
-    unsigned char* dst = w_lds + slot * kWSlot + w * 4096;
+    const unsigned int dst = w_dst0 + slot * kWSlot;
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(wbase + (uint32_t)(w_voff[q] + koff)),
-                                       (lptr_t)(dst + q * 1024), 16, 0, 0);
+      dma16_global_to_lds(wbase, (uint32_t)(w_voff[q] + koff), dst + q * 1024);
   };
   auto issue_x = [&](int kc, int slot) {
     const uint32_t koff = (uint32_t)kc * 128u;
-    unsigned char* dst = x_lds + slot * kXSlot + w * 2048;
+    const unsigned int dst = x_dst0 + slot * kXSlot;
 #pragma unroll
     for (int q = 0; q < 2; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(p.a + (uint32_t)(x_voff[q] + koff)),
-                                       (lptr_t)(dst + q * 1024), 16, 0, 0);
+      dma16_global_to_lds(p.a, (uint32_t)(x_voff[q] + koff), dst + q * 1024);
   };
   // activation scales of chunks [kc0, kc0 + kSC) -> LDS (plain loads; 4 per thread)
   auto load_scales = [&](int kc0) {

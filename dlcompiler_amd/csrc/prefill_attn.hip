@@ -183,10 +183,10 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
       pg_next[i] = bt[p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page)];
     }
   };
+  const unsigned int smem_base = lds_addr(smem) + wave * 1024;  // + q * 1024 with q = 4*i + wave
   auto load_tile = [&](auto clamp_tag, int t0, int buf) {
     constexpr bool CLAMP = decltype(clamp_tag)::value;
-    unsigned char* ks = smem + buf * SM::stage;
-    unsigned char* vs = ks + SM::kBytes;
+    const unsigned int ks = smem_base + buf * SM::stage, vs = ks + SM::kBytes;
     const unsigned char* ksrc[KINS];
     const unsigned char* vsrc[KINS];
 #pragma unroll
@@ -208,9 +208,8 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     }
 #pragma unroll
     for (int i = 0; i < KINS; ++i) {
-      const int q = 4 * i + wave;  // which 1 KB slice of the tile
-      dma16_global_to_lds(ksrc[i], lds_addr(ks + q * 1024));
-      dma16_global_to_lds(vsrc[i], lds_addr(vs + q * 1024));
+      dma16_global_to_lds(ksrc[i], ks + i * 4096);  // 1 KB slice 4*i + wave of the tile
+      dma16_global_to_lds(vsrc[i], vs + i * 4096);
     }
     if (PAGED) fetch_pages(t0 + kTileN);
   };
@@ -257,6 +256,9 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
+    // MFMA-dense phase: let this wave's issue win over the other wave of the SIMD, whose
+    // softmax arithmetic then fills the gaps while the matrix pipe is busy
+    __builtin_amdgcn_s_setprio(1);
     {
       const unsigned char* krow0 = ks + col * SM::kRowBytes;
       const unsigned char* krow1 = ks + (32 + col) * SM::kRowBytes;
@@ -280,6 +282,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
       }
     }
 
+    __builtin_amdgcn_s_setprio(0);
     // ---- causal mask and tile maximum of the raw scores (scale > 0 commutes with max)
     float mloc = -__builtin_inff();
 #pragma unroll
