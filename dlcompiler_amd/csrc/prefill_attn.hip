@@ -184,11 +184,14 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     }
   };
   const unsigned int smem_base = lds_addr(smem) + wave * 1024;  // + q * 1024 with q = 4*i + wave
-  auto load_tile = [&](auto clamp_tag, int t0, int buf) {
+  // source addresses and LDS targets of the copies of the tile being staged: prepare_tile
+  // computes them, issue_copy(n) sends copy n of 2 * KINS (K and V slices alternate)
+  const unsigned char* ksrc[KINS];
+  const unsigned char* vsrc[KINS];
+  unsigned int stage_dst = 0;
+  auto prepare_tile = [&](auto clamp_tag, int t0, int buf) {
     constexpr bool CLAMP = decltype(clamp_tag)::value;
-    const unsigned int ks = smem_base + buf * SM::stage, vs = ks + SM::kBytes;
-    const unsigned char* ksrc[KINS];
-    const unsigned char* vsrc[KINS];
+    stage_dst = smem_base + buf * SM::stage;
 #pragma unroll
     for (int i = 0; i < KINS; ++i) {
       const int r = (4 * i + wave) * KRPI + k_lrow;  // key row inside the tile
@@ -206,12 +209,17 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
       ksrc[i] += (k_pos ^ (r & (DG - 1))) << 4;
       vsrc[i] += (k_pos ^ v_swz(r)) << 4;
     }
+    if (PAGED) fetch_pages(t0 + kTileN);  // consumed by the next prepare_tile
+  };
+  auto issue_copy = [&](int n) {
+    const int i = n >> 1;  // 1 KB slice 4*i + wave of the tile
+    if (n & 1) dma16_global_to_lds(vsrc[i], stage_dst + SM::kBytes + i * 4096);
+    else dma16_global_to_lds(ksrc[i], stage_dst + i * 4096);
+  };
+  auto load_tile = [&](auto clamp_tag, int t0, int buf) {
+    prepare_tile(clamp_tag, t0, buf);
 #pragma unroll
-    for (int i = 0; i < KINS; ++i) {
-      dma16_global_to_lds(ksrc[i], ks + i * 4096);  // 1 KB slice 4*i + wave of the tile
-      dma16_global_to_lds(vsrc[i], vs + i * 4096);
-    }
-    if (PAGED) fetch_pages(t0 + kTileN);
+    for (int n = 0; n < 2 * KINS; ++n) issue_copy(n);
   };
 
   f32x16 o[MT];
@@ -240,8 +248,12 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   }
 
   // one K/V tile against this wave's 32 queries; MASK: apply the causal mask
-  auto process_tile = [&](auto mask_tag, int j) {
+  // COPY: the copies of the tile prepared by prepare_tile go out between the S^T MFMAs, one per
+  // k-step, instead of as one burst that would hold up this wave's instruction stream
+  auto process_tile = [&](auto mask_tag, auto copy_tag, int j) {
     constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr bool COPY = decltype(copy_tag)::value;
+    static_assert(2 * KINS == KS, "one copy per k-step");
     const int t0 = j * kTileN;
     if (MASK && t0 > wave_last_pos) return;  // wave-uniform: tile entirely above the diagonal
     if (MASK && window > 0 && t0 + kTileN - 1 < wave_last_pos - 31 - window) return;  // below the window
@@ -275,6 +287,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
 #pragma unroll
       for (int kstep = 0; kstep < KS; ++kstep) {
         if (kstep + kAhead < KS) ldk(kstep + kAhead, ka[(kstep + kAhead) % (kAhead + 1)]);
+        if (COPY) issue_copy(kstep);
         __builtin_amdgcn_sched_barrier(0);  // keep the fetch ahead of the MFMAs (it would be sunk)
         s[0] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][0], qf[kstep], s[0]);
         s[1] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][1], qf[kstep], s[1]);
@@ -364,9 +377,11 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   __syncthreads();
 
   // tiles under the diagonal whose successor is also under it: nothing to mask or clamp
+  using Yes = std::integral_constant<bool, true>;
+  using No = std::integral_constant<bool, false>;
   for (; j + 1 < nfull; ++j) {
-    load_tile(NoClamp{}, (j + 1) * kTileN, (j + 1) & 1);
-    process_tile(std::integral_constant<bool, false>{}, j);
+    prepare_tile(NoClamp{}, (j + 1) * kTileN, (j + 1) & 1);
+    process_tile(No{}, Yes{}, j);
     wait_dma();
     __syncthreads();
   }
@@ -374,8 +389,8 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   for (; j < ntiles; ++j) {
     const bool more = (j + 1 < ntiles);
     if (more) load_tile(Clamp{}, (j + 1) * kTileN, (j + 1) & 1);
-    if (j < nfull) process_tile(std::integral_constant<bool, false>{}, j);
-    else process_tile(std::integral_constant<bool, true>{}, j);
+    if (j < nfull) process_tile(No{}, No{}, j);
+    else process_tile(Yes{}, No{}, j);
     wait_dma();
     __syncthreads();
   }
