@@ -107,6 +107,13 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// a pointer the caller knows to be wave-uniform, moved into scalar registers
+__device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (const unsigned char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
 // wave-uniform LDS byte address of a pointer into __shared__ memory, in a scalar register
 __device__ __forceinline__ unsigned int lds_addr(const void* p) {
   typedef const __attribute__((address_space(3))) void* lds_ptr_t;

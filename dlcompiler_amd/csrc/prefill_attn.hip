@@ -186,35 +186,58 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   const unsigned int smem_base = lds_addr(smem) + wave * 1024;  // + q * 1024 with q = 4*i + wave
   // source addresses and LDS targets of the copies of the tile being staged: prepare_tile
   // computes them, issue_copy(n) sends copy n of 2 * KINS (K and V slices alternate)
+  // Packed layout: a copy's address is a tile base in scalar registers plus a 32-bit lane
+  // offset that does not change from tile to tile (row inside the tile x row pitch + chunk),
+  // so an unclamped tile costs no vector arithmetic.  Paged layout: every row has its own
+  // page, so full 64-bit lane addresses are formed.
   const unsigned char* ksrc[KINS];
   const unsigned char* vsrc[KINS];
+  unsigned int koff[KINS], voff[KINS], koff0[KINS], voff0[KINS];
+  const unsigned char* kbase = nullptr;
+  const unsigned char* vbase = nullptr;
+#pragma unroll
+  for (int i = 0; i < KINS; ++i) {
+    const int r = (4 * i + wave) * KRPI + k_lrow;
+    koff0[i] = (unsigned int)(r * k_row_bytes) + ((k_pos ^ (r & (DG - 1))) << 4);
+    voff0[i] = (unsigned int)(r * v_row_bytes) + ((k_pos ^ v_swz(r)) << 4);
+  }
   unsigned int stage_dst = 0;
   auto prepare_tile = [&](auto clamp_tag, int t0, int buf) {
     constexpr bool CLAMP = decltype(clamp_tag)::value;
     stage_dst = smem_base + buf * SM::stage;
+    if (!PAGED) {
+      kbase = uniform_ptr(kbytes + (tok0 + t0) * k_row_bytes);
+      vbase = uniform_ptr(vbytes + (tok0 + t0) * v_row_bytes);
+    }
 #pragma unroll
     for (int i = 0; i < KINS; ++i) {
       const int r = (4 * i + wave) * KRPI + k_lrow;  // key row inside the tile
-      int key = t0 + r;
-      if (CLAMP) key = min(key, kv_total - 1);
       if (PAGED) {
+        int key = t0 + r;
+        if (CLAMP) key = min(key, kv_total - 1);
         const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
         const int64_t slot = key - pi * p.page;
-        ksrc[i] = kbytes + ((int64_t)pg_next[i] * p.k_sp + slot * p.k_st) * 2;
-        vsrc[i] = vbytes + ((int64_t)pg_next[i] * p.v_sp + slot * p.v_st) * 2;
+        ksrc[i] = kbytes + ((int64_t)pg_next[i] * p.k_sp + slot * p.k_st) * 2 +
+                  ((k_pos ^ (r & (DG - 1))) << 4);
+        vsrc[i] = vbytes + ((int64_t)pg_next[i] * p.v_sp + slot * p.v_st) * 2 +
+                  ((k_pos ^ v_swz(r)) << 4);
+      } else if (CLAMP) {
+        const int rc = min(r, kv_total - 1 - t0);  // >= 0: a staged tile starts inside the context
+        koff[i] = (unsigned int)(rc * k_row_bytes) + ((k_pos ^ (r & (DG - 1))) << 4);
+        voff[i] = (unsigned int)(rc * v_row_bytes) + ((k_pos ^ v_swz(r)) << 4);
       } else {
-        ksrc[i] = kbytes + (tok0 + key) * k_row_bytes;
-        vsrc[i] = vbytes + (tok0 + key) * v_row_bytes;
+        koff[i] = koff0[i];
+        voff[i] = voff0[i];
       }
-      ksrc[i] += (k_pos ^ (r & (DG - 1))) << 4;
-      vsrc[i] += (k_pos ^ v_swz(r)) << 4;
     }
     if (PAGED) fetch_pages(t0 + kTileN);  // consumed by the next prepare_tile
   };
   auto issue_copy = [&](int n) {
     const int i = n >> 1;  // 1 KB slice 4*i + wave of the tile
-    if (n & 1) dma16_global_to_lds(vsrc[i], stage_dst + SM::kBytes + i * 4096);
-    else dma16_global_to_lds(ksrc[i], stage_dst + i * 4096);
+    const unsigned int dst = stage_dst + (n & 1) * SM::kBytes + i * 4096;
+    if (PAGED) dma16_global_to_lds((n & 1) ? vsrc[i] : ksrc[i], dst);
+    else if (n & 1) dma16_global_to_lds(vbase, voff[i], dst);
+    else dma16_global_to_lds(kbase, koff[i], dst);
   };
   auto load_tile = [&](auto clamp_tag, int t0, int buf) {
     prepare_tile(clamp_tag, t0, buf);
