@@ -412,7 +412,9 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   for (; j < ntiles; ++j) {
     const bool more = (j + 1 < ntiles);
     if (more) load_tile(Clamp{}, (j + 1) * kTileN, (j + 1) & 1);
-    if (j < nfull) process_tile(No{}, No{}, j);
+    // a diagonal tile still lies entirely under the diagonal for the waves further down
+    const bool wave_full = !generic && (j + 1) * kTileN - 1 <= hist + q0 + 32 * wave;
+    if (j < nfull || wave_full) process_tile(No{}, No{}, j);
     else process_tile(Yes{}, No{}, j);
     wait_dma();
     __syncthreads();
