@@ -261,7 +261,10 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   u32x4 areg[AU];
   float asreg = 0.0f;
   i32x8 breg[PD][4];
-  float bsreg[PD][4];
+  // block scales of a wave's sub-tiles: sub-tiles 0,1 and 2,3 share a 128-column block (gate /
+  // up columns; one block for all four in the down GEMM)
+  constexpr int NSC = GATED ? 2 : 1;
+  float bsreg[PD][NSC];
   const int NS = (KC + SKC - 1) / SKC;
 
   auto load_a = [&](int st) {  // stage st -> registers (chunks past K are clamped, unused)
@@ -279,7 +282,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     for (int u = 0; u < AU; ++u) *(u32x4*)(dst + (u % RP) * 32 * kARow + (u / RP) * 128) = areg[u];
     if (QT == 0 && aseg < SKC) as_lds[buf][aseg][arow] = asreg;
   };
-  auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[4]) {
+  auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[NSC]) {
     if (kc >= KC) return;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -288,18 +291,18 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
       const u32x4 hi = *(const u32x4*)(src + w_hi_off + woff[j]);
       b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
                    (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-      bs[j] = QT == 0 ? ws_ptr[j][kc] : 1.0f;
     }
+#pragma unroll
+    for (int q = 0; q < NSC; ++q) bs[q] = QT == 0 ? ws_ptr[2 * q][kc] : 1.0f;
   };
 
   // software pipeline state: products of the previous 16-token step and their scales
   f32x4 pp[4];
-  float psc[4];
+  float psc[NSC];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    pp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    psc[j] = 0.0f;
-  }
+  for (int j = 0; j < 4; ++j) pp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int q = 0; q < NSC; ++q) psc[q] = 0.0f;
   // A stage is SKC * MT steps of 16 tokens x one chunk.  Step t issues its 4 MFMAs, each
   // followed by the FMAs that retire one product of step t - 1 (for the first step of a
   // stage: the last step of the previous stage); the activation fragment of step t + 1 is
@@ -343,16 +346,15 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               pc[j] = mfma_fp8(breg[slot][j], xq[t & 1]);
-              acc[pm][j] += pp[j] * psc[j];
+              acc[pm][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
             }
             // keep the retiring FMAs next to these MFMAs (the optimiser would otherwise sink
             // them into one long VALU run with nothing to overlap)
             asm volatile("" : "+v"(acc[pm][0]), "+v"(acc[pm][1]), "+v"(acc[pm][2]), "+v"(acc[pm][3]));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              pp[j] = pc[j];
-              psc[j] = asq[t & 1] * bsreg[slot][j];
-            }
+            for (int j = 0; j < 4; ++j) pp[j] = pc[j];
+#pragma unroll
+            for (int q = 0; q < NSC; ++q) psc[q] = asq[t & 1] * bsreg[slot][q];
           } else {
             (void)pm;
 #pragma unroll
@@ -380,7 +382,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   }
   // retire the products of the very last step
 #pragma unroll
-  for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[j];
+  for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
 
   // ---- epilogues: lane holds token (16*mt + c), columns ncol[j] + 4*g + i
   if (GATED && QT == 1) {
