@@ -131,6 +131,34 @@ def wl_silu(dev, steps, warmup, cpu):
     return res
 
 
+def _graph_replay_ms(fn, steps, warmup, label):
+    """Mean time of one replay of ``fn`` captured into a HIP graph (optional extra figure: the
+    public calls with no Python or launch latency between their kernels).  None if capture fails."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            out = fn()
+        for _ in range(warmup):
+            g.replay()
+        torch.cuda.synchronize()
+        t = Timer()
+        ev = t.start()
+        for _ in range(steps):
+            g.replay()
+        t.stop(ev)
+        ms = t.mean_ms() / steps
+        del out, g
+        return ms
+    except Exception as exc:  # graph capture is optional reporting
+        print(f"[bench] {label} graph replay skipped: {exc}", file=sys.stderr)
+        return None
+
+
 def wl_gating(dev, steps, warmup, cpu):
     from dlcompiler_amd.kernels.moe_gating import moe_align_block_size, moe_topk_softmax
 
@@ -148,29 +176,7 @@ def wl_gating(dev, steps, warmup, cpu):
     ms, _ = _time_steps(step, steps, warmup)
 
     # the same two calls replayed from a HIP graph (no Python / launch latency in between)
-    graph_ms = None
-    try:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step(0)
-        torch.cuda.current_stream().wait_stream(side)
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            out = step(0)
-        for _ in range(warmup):
-            g.replay()
-        torch.cuda.synchronize()
-        t = Timer()
-        ev = t.start()
-        for _ in range(steps):
-            g.replay()
-        t.stop(ev)
-        graph_ms = t.mean_ms() / steps
-        del out
-    except Exception as exc:  # graph capture is optional reporting
-        graph_ms = None
-        print(f"[bench] gating graph replay skipped: {exc}", file=sys.stderr)
+    graph_ms = _graph_replay_ms(lambda: step(0), steps, warmup, "gating")
 
     # dominant kernel: the router (reads the logits, 72% of the bytes)
     tk = Timer()
@@ -339,6 +345,9 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
     ms, _ = _time_steps(lambda i: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled),
                         steps, warmup)
 
+    graph_ms = _graph_replay_ms(
+        lambda: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled), steps, warmup, "moe")
+
     stage_t = {}
     state = {"name": None, "ev": None}
 
@@ -361,6 +370,8 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
                    "weight_layout": "operand-order" if shuffled else "row-major",
                    "algorithmic_flops": flops},
         "stages_ms": stages,
+        "graph_replay": None if graph_ms is None else {
+            "ms_per_step": graph_ms, "value": flops / graph_ms / 1e9, "unit": "TFLOP/s"},
         "gemm_only_tflops": flops / (stages["gate_up"] + stages["down"]) / 1e9,
         "roofline": {"kernel": "moe_gemm_fp8_kernel<gate_up>", "bound": "mfma",
                      "achieved": gate_up_flops / ms_gate_up / 1e9, "peak": PEAK_FP8_TFLOPS,
