@@ -154,6 +154,15 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
   return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p));
 }
 
+// max of a value and its partner 32 lanes away (v_permlane32_swap: a register-file exchange,
+// no trip through LDS as with ds_bpermute)
+__device__ __forceinline__ float max_xor32(float v) {
+  typedef __attribute__((ext_vector_type(2))) unsigned int u2;
+  const unsigned int u = __float_as_uint(v);
+  const u2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) {
   return (a + b - 1) / b;
 }

@@ -320,7 +320,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
 
     __builtin_amdgcn_s_setprio(0);
     // ---- causal mask and tile maximum of the raw scores (scale > 0 commutes with max)
-    float mloc = -__builtin_inff();
+    float mpart[2] = {-__builtin_inff(), -__builtin_inff()};  // two independent chains
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
@@ -334,10 +334,10 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
           if (window > 0) vis = vis && (key >= qpos - window);
           s[nt][i] = vis ? x : -__builtin_inff();
         }
-        mloc = fmaxf(mloc, s[nt][i]);
+        mpart[nt] = fmaxf(mpart[nt], s[nt][i]);
       }
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * cs;
+    const float mloc = max_xor32(fmaxf(mpart[0], mpart[1])) * cs;
     if (__any(mloc > m_run + kRescaleGap)) {
       const float m_new = fmaxf(m_run, mloc);  // finite from tile 0 on (key 0 is visible)
       // (a fully masked row under a sliding window keeps m_new = -inf: leave it untouched)
