@@ -119,6 +119,10 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
     for (int d = 32; d >= 1; d >>= 1) t += __shfl_xor(t, d);
     total += t;
   }
+  // (the reduction leaves the same value in every lane; say so, or every address derived from
+  // it is treated as lane-dependent and the block-table lookups become vector loads that
+  // share the in-order return queue of the K/V stream)
+  total = __builtin_amdgcn_readfirstlane(total);
   const int upt = max((total + p.num_teams - 1) / p.num_teams, p.min_units);  // units per team
   const int lo = team * upt;
   if (lo >= total) return;
@@ -126,6 +130,7 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
 
   // one sequence segment [k_begin, k_end) of sequence b -> partial number `piece` of b
   auto process_segment = [&](int b, int k_begin, int k_end, int piece) {
+  b = __builtin_amdgcn_readfirstlane(b);
   const int ctx = p.kv_len[b];
   k_end = min(k_end, ctx);
   const int kv_min = p.window > 0 ? max(ctx - 1 - p.window, 0) : 0;  // first visible key
@@ -165,12 +170,35 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
     u32x4 kf[2][KS];          // K: 2 sub-tiles of 16 keys, already in A-operand layout
     u32x4 vr[2][VPASS][4];    // V: per lane 4 consecutive keys x 8 dims per pass
   };
+  // Block-table lookups are wave-uniform and must be SCALAR loads: as vector loads they sit in
+  // the same in-order return queue as the K/V stream, and waiting for a page number means
+  // waiting for every half tile still in flight.  The compiler will not use the scalar path for
+  // memory the kernel might have written, so the load is issued by hand (and waited for on
+  // the scalar counter), one half tile ahead of the loads that need the page numbers.
+  int pg_ahead[2];  // physical pages of the two 16-key sub-tiles of the next half tile to load
+  auto lookup_pages = [&](int h0) {
+    const int32_t* entry[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      const int base_key = min(h0 + 16 * sub, ctx - 1);  // clamp: never look past the context
+      const int pi = POW2 ? (base_key >> p.page_shift) : (base_key / p.page);
+      entry[sub] = (const int32_t*)uniform_ptr((const unsigned char*)(bt + pi));
+    }
+    int p0, p1;
+    asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(p0), "=&s"(p1)
+                 : "s"(entry[0]), "s"(entry[1]));
+    pg_ahead[0] = p0;
+    pg_ahead[1] = p1;
+  };
   auto load_half = [&](int h0, HalfTile& f) {
+    const int pg_now[2] = {pg_ahead[0], pg_ahead[1]};
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       const int base_key = min(h0 + 16 * sub, ctx - 1);  // uniform; clamp: never read past ctx
-      const int pi = POW2 ? (base_key >> p.page_shift) : (base_key / p.page);
-      const int64_t pg = (int64_t)bt[pi];
+      const int pi =
+          __builtin_amdgcn_readfirstlane(POW2 ? (base_key >> p.page_shift) : (base_key / p.page));
+      const int64_t pg = (int64_t)pg_now[sub];
       const int page_key0 = pi * p.page;
       {
         const int key = min(h0 + 16 * sub + c, ctx - 1);
@@ -197,6 +225,7 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
         }
       }
     }
+    lookup_pages(h0 + 32);
   };
   // st = parity of the half tile inside its 64-key tile = which 4 units of a V^T row it uses
   auto compute_half = [&](int h0, const HalfTile& f, int st) {
@@ -291,19 +320,30 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
   };
 
   HalfTile ha, hb;
-  if (k_begin < k_end) load_half(k_begin, ha);  // (a segment entirely before the window is empty)
-  for (int t0 = k_begin; t0 < k_end; t0 += kTile) {
-    const bool second = t0 + 32 < k_end;
-    if (second) load_half(t0 + 32, hb);
-    __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic below
-    compute_half(t0, ha, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (second) {
-      if (t0 + kTile < k_end) load_half(t0 + kTile, ha);
+  if (k_begin < k_end) {  // (a segment entirely before the window is empty)
+    lookup_pages(k_begin);
+    load_half(k_begin, ha);
+    int t0 = k_begin;
+    // steady state: the tile has both halves and another tile follows.  No run-time condition
+    // surrounds a load here: where the two paths of a branch around loads join, the compiler
+    // has to wait as if the loads had not been issued, i.e. for the ones just sent.
+    for (; t0 + kTile < k_end; t0 += kTile) {
+      load_half(t0 + 32, hb);
+      __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic below
+      compute_half(t0, ha, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      load_half(t0 + kTile, ha);
       __builtin_amdgcn_sched_barrier(0);
       compute_half(t0 + 32, hb, 1);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // last tile: one or two halves
+    const bool second = t0 + 32 < k_end;
+    if (second) load_half(t0 + 32, hb);
+    __builtin_amdgcn_sched_barrier(0);
+    compute_half(t0, ha, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (second) compute_half(t0 + 32, hb, 1);
   }
 
   l_run += __shfl_xor(l_run, 16);
