@@ -265,15 +265,24 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
 
     // ---- online softmax over these 32 keys (log2 domain) ----
     float mloc = -__builtin_inff();
+    if (p.softcap > 0.0f) {  // one uniform branch for the half tile, not one per element
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          s[sub][i] = p.softcap * tanhf(s[sub][i] * p.sm_scale / p.softcap) * 1.4426950408889634f;
+    } else {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[sub][i] *= p.scale_log2e;
+    }
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = h0 + 16 * sub + 4 * g + i;
-        float x = s[sub][i] * p.scale_log2e;
-        if (p.softcap > 0.0f)
-          x = p.softcap * tanhf(s[sub][i] * p.sm_scale / p.softcap) * 1.4426950408889634f;
-        x = (key < k_end && key >= kv_min) ? x : -__builtin_inff();
+        const float x = (key < k_end && key >= kv_min) ? s[sub][i] : -__builtin_inff();
         s[sub][i] = x;
         mloc = fmaxf(mloc, x);
       }
