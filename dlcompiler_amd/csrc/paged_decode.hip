@@ -130,11 +130,13 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
 
   // one sequence segment [k_begin, k_end) of sequence b -> partial number `piece` of b
   auto process_segment = [&](int b, int k_begin, int k_end, int piece) {
+  // everything that shapes the walk is wave-uniform; saying so keeps the loops and the page
+  // arithmetic on the scalar unit
   b = __builtin_amdgcn_readfirstlane(b);
-  const int ctx = p.kv_len[b];
-  k_end = min(k_end, ctx);
+  const int ctx = __builtin_amdgcn_readfirstlane(p.kv_len[b]);
+  k_end = __builtin_amdgcn_readfirstlane(min(k_end, ctx));
   const int kv_min = p.window > 0 ? max(ctx - 1 - p.window, 0) : 0;  // first visible key
-  k_begin = max(k_begin, kv_min & ~31);  // start at the half tile that holds kv_min
+  k_begin = __builtin_amdgcn_readfirstlane(max(k_begin, kv_min & ~31));  // the half tile holding kv_min
   const int32_t* bt = p.block_table + (int64_t)b * p.bt_stride;
 
   // Q^T as the B operand: lane (n = query head c, k = dims 32*ks + 8g .. +8)
