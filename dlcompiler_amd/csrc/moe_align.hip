@@ -10,6 +10,8 @@
 //   2. scan:   one workgroup turns the [chunks, E] table into per-chunk start offsets, pads each
 //              expert's total to `block`, and emits counts, block -> expert ids, the sentinel
 //              pad slots and the padded total;
+//      (for up to 256 chunks step 2 is folded into step 3: every workgroup reduces the small
+//      count table itself, which saves a launch on the sizes a decoder layer produces)
 //   3. place:  every workgroup re-reads its chunk in order and writes flat index i to
 //              start[chunk][e] + (number of earlier i' in the chunk with the same e), the rank
 //              coming from wave ballots, which makes the sort stable (ascending i per expert).
@@ -176,6 +178,116 @@ __global__ __launch_bounds__(kThreads) void align_place_kernel(
   }
 }
 
+// Scan and placement in one launch, for inputs of up to kFusedChunks chunks: every workgroup
+// reduces the (small) [chunks, E] count table itself -- expert totals, padded expert bases and
+// the offsets of its own chunk -- instead of waiting for a separate one-workgroup scan kernel;
+// workgroup 0 also emits what the scan kernel emits (counts, block -> expert ids, pad slots,
+// tails, padded total).  The table is only read here.
+constexpr int kFusedChunks = 256;
+
+__global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
+    const int32_t* __restrict__ ids, int64_t numel, int E, int block,
+    const int32_t* __restrict__ chunk_counts, int chunks, int32_t* __restrict__ sorted_ids,
+    int64_t sorted_cap, int32_t* __restrict__ expert_ids, int64_t expert_ids_cap,
+    int32_t* __restrict__ counts, int32_t* __restrict__ num_post_pad) {
+  __shared__ int32_t cursor[kMaxE];            // next free slot per expert for this chunk
+  __shared__ int32_t wave_cnt[kWaves][kMaxE];  // per-tile, per-wave counts
+  __shared__ int32_t total_s[kMaxE];
+  __shared__ int32_t base_s[kMaxE + 1];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int me = blockIdx.x;
+
+  // totals and the part of them that lies in earlier chunks (thread e <-> expert e)
+  int32_t before = 0;
+  if (tid < E) {
+    int32_t total = 0;
+    for (int c = 0; c < chunks; ++c) {
+      const int32_t n = chunk_counts[(int64_t)c * E + tid];
+      total += n;
+      if (c < me) before += n;
+    }
+    total_s[tid] = total;
+  }
+  for (int i = tid; i < kWaves * kMaxE; i += kThreads) (&wave_cnt[0][0])[i] = 0;
+  __syncthreads();
+  if (tid < 64) {  // padded totals -> expert bases: wave scan over up to 256 experts
+    int32_t run = 0;
+    for (int i0 = 0; i0 < E; i0 += 64) {
+      const int i = i0 + tid;
+      const int32_t padded = (i < E) ? (int32_t)(ceil_div(total_s[i], block) * block) : 0;
+      int32_t incl = padded;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d);
+        if (tid >= d) incl += up;
+      }
+      if (i < E) base_s[i] = run + incl - padded;
+      run += __shfl(incl, 63);
+    }
+    if (tid == 0) base_s[E] = run;
+  }
+  __syncthreads();
+  if (tid < E) cursor[tid] = base_s[tid] + before;
+  if (me == 0) {
+    const int32_t total_padded = base_s[E];
+    if (tid == 0) *num_post_pad = total_padded;
+    if (tid < E) {
+      const int32_t base = base_s[tid], total = total_s[tid], next = base_s[tid + 1];
+      if (counts) counts[tid] = total;
+      for (int32_t q = base + total; q < next; ++q) sorted_ids[q] = (int32_t)numel;  // pad slots
+      for (int32_t b = base / block; b < next / block; ++b) expert_ids[b] = tid;
+    }
+    for (int64_t q = (int64_t)total_padded + tid; q < sorted_cap; q += kThreads)
+      sorted_ids[q] = (int32_t)numel;
+    for (int64_t b = (int64_t)total_padded / block + tid; b < expert_ids_cap; b += kThreads)
+      expert_ids[b] = -1;
+  }
+  __syncthreads();
+
+  const int64_t begin = (int64_t)me * kChunk;
+  const int64_t end = begin + kChunk < numel ? begin + kChunk : numel;
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int64_t tile = begin; tile < end; tile += kThreads) {  // uniform trip count
+    const int64_t i = tile + tid;
+    int32_t e = -1;
+    if (i < end) {
+      e = ids[i];
+      if (e < 0 || e >= E) e = -1;
+    }
+    // lanes of this wave holding the same expert: intersect ballots over the 9 key bits
+    const uint32_t key = (uint32_t)e & 0x1ffu;
+    uint64_t peers = ~0ull;
+#pragma unroll
+    for (int b = 0; b < 9; ++b) {
+      const bool bit = (key >> b) & 1u;
+      const uint64_t m = __ballot(bit);
+      peers &= bit ? m : ~m;
+    }
+    const int rank_in_wave = __popcll(peers & lt_mask);
+    const int peer_count = __popcll(peers);
+    if (e >= 0 && rank_in_wave == 0) wave_cnt[wave][e] = peer_count;
+    __syncthreads();
+    if (e >= 0) {
+      int32_t pos = cursor[e] + rank_in_wave;
+      for (int w = 0; w < wave; ++w) pos += wave_cnt[w][e];
+      sorted_ids[pos] = (int32_t)i;
+    }
+    __syncthreads();
+    for (int x = tid; x < E; x += kThreads) {
+      int32_t add = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        add += wave_cnt[w][x];
+        wave_cnt[w][x] = 0;
+      }
+      cursor[x] += add;
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace
 }  // namespace dlb
 
@@ -203,6 +315,13 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
   int32_t* chunk_counts = (int32_t*)ws;
   hipLaunchKernelGGL(align_count_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
                      numel, E, chunk_counts);
+  if (chunks <= kFusedChunks) {
+    // (with numel = 0 the single chunk is empty: workgroup 0 still writes pads, tails and totals)
+    hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s,
+                       topk_ids, numel, E, block, chunk_counts, (int)chunks, sorted_ids, sorted_cap,
+                       expert_ids, expert_ids_cap, counts, num_post_pad);
+    return launch_status();
+  }
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, chunk_counts, chunks, E, block,
                      (int32_t)numel, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, counts,
                      num_post_pad);

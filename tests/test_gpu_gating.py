@@ -69,7 +69,8 @@ def _align(ids_cpu, block, E, dev):
 
 @pytest.mark.parametrize("T,k,E,block", [(16384, 6, 64, 64), (4096, 6, 64, 64), (128, 2, 4, 16),
                                          (1, 6, 64, 64), (7, 3, 5, 1), (1000, 8, 256, 128),
-                                         (3000, 4, 60, 32), (2048, 1, 2, 64), (513, 2, 160, 8)])
+                                         (3000, 4, 60, 32), (2048, 1, 2, 64), (513, 2, 160, 8),
+                                         (140000, 4, 32, 64)])  # > 256 chunks: separate scan kernel
 def test_align_bit_exact(dev, T, k, E, block):
     g = torch.Generator().manual_seed(1)
     logits = torch.randn((T, E), generator=g)
