@@ -199,17 +199,41 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   const int wave = tid / kWave;
   const int me = blockIdx.x;
 
-  // totals and the part of them that lies in earlier chunks (thread e <-> expert e)
+  // totals and the part of them that lies in earlier chunks: sub-group q = tid / E' (E' = E
+  // rounded up to a whole wave) sums a slice of the chunk rows for expert tid % E', the slices
+  // meet in LDS (wave_cnt doubles as the scratch for that before it is cleared)
+  const int ep = (E + 63) & ~63;
+  const int groups = kThreads / ep;  // 4, 2 or 1
+  {
+    const int e = tid % ep, q = tid / ep;
+    const int per = (chunks + groups - 1) / groups;
+    const int c0 = q * per, c1 = min(c0 + per, chunks);
+    int32_t total = 0, before_part = 0;
+    if (e < E && q < groups) {
+      for (int c = c0; c < c1; ++c) {
+        const int32_t n = chunk_counts[(int64_t)c * E + e];
+        total += n;
+        if (c < me) before_part += n;
+      }
+    }
+    int32_t* part = &wave_cnt[0][0];  // [2][groups][ep] <= 2 * 256 entries
+    if (q < groups) {
+      part[q * ep + e] = total;
+      part[kThreads + q * ep + e] = before_part;
+    }
+  }
+  __syncthreads();
   int32_t before = 0;
   if (tid < E) {
+    const int32_t* part = &wave_cnt[0][0];
     int32_t total = 0;
-    for (int c = 0; c < chunks; ++c) {
-      const int32_t n = chunk_counts[(int64_t)c * E + tid];
-      total += n;
-      if (c < me) before += n;
+    for (int q = 0; q < groups; ++q) {
+      total += part[q * ep + tid];
+      before += part[kThreads + q * ep + tid];
     }
     total_s[tid] = total;
   }
+  __syncthreads();
   for (int i = tid; i < kWaves * kMaxE; i += kThreads) (&wave_cnt[0][0])[i] = 0;
   __syncthreads();
   if (tid < 64) {  // padded totals -> expert bases: wave scan over up to 256 experts
