@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kThreads) void align_place_kernel(
 // Scan and placement in one launch, for inputs of up to kFusedChunks chunks: every workgroup
 // reduces the (small) [chunks, E] count table itself -- expert totals, padded expert bases and
 // the offsets of its own chunk -- instead of waiting for a separate one-workgroup scan kernel;
-// workgroup 0 also emits what the scan kernel emits (counts, block -> expert ids, pad slots,
+// one extra workgroup emits what the scan kernel emits (counts, block -> expert ids, pad slots,
 // tails, padded total).  The table is only read here.
 constexpr int kFusedChunks = 256;
 
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   }
   __syncthreads();
   if (tid < E) cursor[tid] = base_s[tid] + before;
-  if (me == 0) {
+  if (me == chunks) {  // the extra workgroup: what the scan kernel emits besides offsets
     const int32_t total_padded = base_s[E];
     if (tid == 0) *num_post_pad = total_padded;
     if (tid < E) {
@@ -267,6 +267,7 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
       sorted_ids[q] = (int32_t)numel;
     for (int64_t b = (int64_t)total_padded / block + tid; b < expert_ids_cap; b += kThreads)
       expert_ids[b] = -1;
+    return;
   }
   __syncthreads();
 
@@ -340,8 +341,8 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
   hipLaunchKernelGGL(align_count_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
                      numel, E, chunk_counts);
   if (chunks <= kFusedChunks) {
-    // (with numel = 0 the single chunk is empty: workgroup 0 still writes pads, tails and totals)
-    hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s,
+    // (with numel = 0 the single chunk is empty: the extra workgroup still writes pads, tails and totals)
+    hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s,
                        topk_ids, numel, E, block, chunk_counts, (int)chunks, sorted_ids, sorted_cap,
                        expert_ids, expert_ids_cap, counts, num_post_pad);
     return launch_status();
