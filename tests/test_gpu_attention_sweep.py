@@ -1,0 +1,89 @@
+"""GPU parity: seeded random-shape sweeps of the three attention entry points against the CPU
+oracle (ragged lengths around the tile sizes, odd page sizes, GQA ratios, window, soft-cap)."""
+import random
+
+import pytest
+import torch
+
+from oracle import attention as oa
+
+pytestmark = pytest.mark.gpu
+
+_LENS = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 257]
+
+
+def _close(out, ref):
+    out = out.float()
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out, ref.float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_prefill_sweep(dev, seed):
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    rng = random.Random(100 + seed)
+    d = rng.choice([64, 128])
+    hkv = rng.choice([1, 2, 4])
+    hq = hkv * rng.choice([1, 2, 4])
+    dtype = rng.choice([torch.bfloat16, torch.float16])
+    nseq = rng.randint(1, 4)
+    lens = [rng.choice(_LENS + [rng.randint(1, 700)]) for _ in range(nseq)]
+    gen = torch.Generator().manual_seed(1000 + seed)
+    T = sum(lens)
+    q = torch.randn((T, hq, d), generator=gen).to(dtype)
+    k = torch.randn((T, hkv, d), generator=gen).to(dtype)
+    v = torch.randn((T, hkv, d), generator=gen).to(dtype)
+    start = torch.tensor([sum(lens[:i]) for i in range(nseq)], dtype=torch.int32)
+    sl = torch.tensor(lens, dtype=torch.int32)
+    o = torch.zeros_like(q, device=dev)
+    context_attention_fwd(q.to(dev), k.to(dev), v.to(dev), o, start.to(dev), sl.to(dev), max(lens))
+    _close(o.cpu(), oa.prefill_attention(q, k, v, start, sl))
+
+    # the same queries after a history, through the paged cache
+    page = rng.choice([16, 20, 32, 48, 64, 128])
+    if T == nseq:
+        page = rng.choice([16, 32, 64])  # one token per sequence takes the decode branch
+    hist = [rng.choice([0, 1, 17, 64, 100, rng.randint(0, 500)]) for _ in range(nseq)]
+    full = [a + b for a, b in zip(lens, hist)]
+    ks = [torch.randn((n, hkv, d), generator=gen).to(dtype) for n in full]
+    vs = [torch.randn((n, hkv, d), generator=gen).to(dtype) for n in full]
+    kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=seed, dtype=dtype)
+    window = rng.choice([None, None, 16, 100])
+    softcap = rng.choice([None, None, 30.0])
+    ql, kl = torch.tensor(lens), torch.tensor(full)
+    o2 = torch.zeros_like(q, device=dev)
+    paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o2, table.to(dev), start.to(dev),
+                        ql.to(dev), kl.to(dev), max(lens), window_size=window,
+                        logit_softcapping=softcap)
+    _close(o2.cpu(), oa.paged_prefill(q, kc, vc, table, start.long(), ql, kl, window=window,
+                                      softcap=softcap))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_sweep(dev, seed):
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+
+    rng = random.Random(200 + seed)
+    d = rng.choice([64, 128])
+    hkv = rng.choice([1, 2, 8])
+    hq = hkv * rng.choice([1, 4, 8, 16])
+    dtype = rng.choice([torch.bfloat16, torch.float16])
+    B = rng.choice([1, 2, 5, 17, 64])
+    page = rng.choice([16, 32, 48, 64, 128])
+    ctx = [rng.choice([1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 129, 500, rng.randint(1, 3000)])
+           for _ in range(B)]
+    gen = torch.Generator().manual_seed(2000 + seed)
+    ks = [torch.randn((n, hkv, d), generator=gen).to(dtype) for n in ctx]
+    vs = [torch.randn((n, hkv, d), generator=gen).to(dtype) for n in ctx]
+    kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=seed, dtype=dtype)
+    q = torch.randn((B, hq, d), generator=gen).to(dtype)
+    window = rng.choice([None, None, 16, 100])
+    softcap = rng.choice([None, None, 30.0])
+    kl = torch.tensor(ctx)
+    o = torch.zeros_like(q, device=dev)
+    paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(dev),
+                        torch.arange(B, device=dev), torch.ones(B, dtype=torch.int64, device=dev),
+                        kl.to(dev), 1, window_size=window, logit_softcapping=softcap)
+    _close(o.cpu(), oa.paged_decode(q, kc, vc, table, kl, window=window, softcap=softcap))
