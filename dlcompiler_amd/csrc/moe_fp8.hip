@@ -148,18 +148,53 @@ __device__ __forceinline__ f32x4 mfma_16bit(const i32x8& a, const i32x8& b, f32x
 // GATED = true : gate_up GEMM (N = 2I), tile = 128 gate cols + the matching 128 up cols,
 //                epilogue silu(gate) * up -> fp8 + per-128 scale, rows kept in sorted order.
 // GATED = false: down GEMM, tile = 256 cols, epilogue * routing weight -> out[slot, n].
-// BM = rows (routing slots) per workgroup = the alignment block of the routing (64 or 128).
+// BM = rows (routing slots) per workgroup = the alignment block of the routing.
+//
+// MFMA shape: 32x32x64 (fp8) / 32x32x16 (16 bit).  A wave owns 64 output columns (two 32-column
+// tiles; gated: 32 gate + the matching 32 up columns) x the 64 rows (two 32-row tiles).  Lane
+// (j = lane % 32, h = lane / 32) supplies, for weight row / token j, the four 16-byte pieces
+// q = 0..3 of a 128-byte K chunk at chunk offset 32 q + 16 h; the fp8 MFMA m consumes pieces
+// 2m and 2m + 1, the 16-bit MFMA q consumes piece q.  Its 16 accumulators of a tile are
+// token j, columns 8 (r / 4) + 4 h + r % 4.  The 32x32 shape matters for the fp8 path: next to
+// an fp8 32x32x64 MFMA (64 cycles) the vector ALU retires the 8 scale-and-accumulate FMAs it
+// owes per MFMA at ~94 % matrix-pipe occupancy, next to the 16x16x128 form (32 cycles, 4 FMAs)
+// only at ~70 %.
 #ifndef DLB_MOE_OCC
 #define DLB_MOE_OCC 2
 #endif
-template <bool GATED, int DT, int BM, int QT>
-__device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const int logical) {
-  constexpr int kBM = BM;
-  constexpr int MT = BM / 16;          // 16-token sub-tiles
-  constexpr int SKC = 2;               // 128-byte K chunks per activation stage
 #ifndef DLB_MOE_PD
 #define DLB_MOE_PD 2
 #endif
+
+#ifdef DLB_TIMING
+__device__ unsigned long long dbg_t[4096];
+__device__ int dbg_n;
+#define DLB_T() do { if ((blockIdx.x & 511) == 8 && threadIdx.x == 0 && dbg_n < 2040) { dbg_t[2 * dbg_n] = clock64(); dbg_t[2 * dbg_n + 1] = wall_clock64(); ++dbg_n; } } while (0)
+#else
+#define DLB_T() do { } while (0)
+#endif
+
+__device__ __forceinline__ i32x8 cat8(const u32x4& lo, const u32x4& hi) {
+  return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
+               (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+}
+
+// exchange between the two lane halves: afterwards lane half 0 holds (its a, the partner's a)
+// and lane half 1 (the partner's b, its b), partner = the lane 32 away
+__device__ __forceinline__ void swap_halves(unsigned int& a, unsigned int& b) {
+  typedef __attribute__((ext_vector_type(2))) unsigned int u2;
+  const u2 r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  a = r[0];
+  b = r[1];
+}
+
+template <bool GATED, int DT, int BM, int QT>
+__device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const int logical) {
+  static_assert(BM == 64, "two 32-row MFMA tiles per workgroup");
+  constexpr int kBM = BM;
+  constexpr int RT = BM / 32;          // 32-token row tiles
+  constexpr int CT = 2;                // 32-column tiles per wave
+  constexpr int SKC = 2;               // 128-byte K chunks per activation stage
   constexpr int PD = DLB_MOE_PD;       // weight-fragment ring depth (chunks in flight + 1)
   constexpr int TPR = 256 / BM;        // staging threads per activation row
   constexpr int AU = SKC * 8 / TPR;    // 16-byte units per staging thread and stage
@@ -179,13 +214,13 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
-  const int g = lane >> 4;
-  const int c = lane & 15;
+  const int h = lane >> 5;
+  const int j = lane & 31;
   const int row0 = mb * kBM;
   const int K = p.K, KC = p.KC;
 
+  DLB_T();
   if (tid < kBM) sid_lds[tid] = p.sorted_ids[row0 + tid];
-  static_assert(BM == 64 || BM == 128, "BM");
   static_assert(AU == SKC * (BM / 32), "staging units per thread");
 
   // ---- activation chunk staging.  Data: 8 consecutive lanes fetch one row's 128-byte chunk
@@ -209,60 +244,64 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     as_ptr = QT == 0 ? p.a_scale + src_row_of(arow) * KC : nullptr;
   }
 
-  // ---- weight fragments: sub-tile j of this wave covers 16 output columns
-  int ncol[4];   // first column of sub-tile j in the expert's [N, K] matrix
-  int sblk[4];   // its 128-row scale block
+  // ---- weight fragments: column tile ct of this wave covers 32 output columns
+  int ncol[CT];  // first column of tile ct in the expert's [N, K] matrix
   if (GATED) {
-    const int n0 = nt * 128 + wave * 32;
-    ncol[0] = n0;
-    ncol[1] = n0 + 16;
-    ncol[2] = p.I + n0;
-    ncol[3] = p.I + n0 + 16;
+    ncol[0] = nt * 128 + wave * 32;
+    ncol[1] = p.I + ncol[0];
   } else {
-    const int n0 = nt * 256 + wave * 64;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ncol[j] = n0 + 16 * j;
+    ncol[0] = nt * 256 + wave * 64;
+    ncol[1] = ncol[0] + 32;
   }
   // Weight addressing: one wave-uniform base per expert (kept in scalar registers) plus a
-  // 32-bit per-lane byte offset per sub-tile; the block scales of a sub-tile are wave-uniform
-  // and come through scalar loads.
+  // 32-bit per-lane byte offset per tile; the block scales of a tile are wave-uniform and come
+  // through scalar loads.
   const unsigned char* wbase = p.w + (int64_t)e * p.N * K;
-  uint32_t woff[4];
-  const float* ws_ptr[4];
-  // byte distance between consecutive K chunks / between the two 16-byte operand halves
+  uint32_t woff[CT];
+  const float* ws_ptr[CT];
+  // byte distance between consecutive K chunks / between the four pieces of a lane
   const int w_kc_stride = p.w_layout ? 2048 : 128;
-  const int w_hi_off = p.w_layout ? 1024 : 64;
+  const int w_q_stride = p.w_layout ? 512 : 32;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    sblk[j] = __builtin_amdgcn_readfirstlane(min(ncol[j] >> 7, (p.N >> 7) - 1));
+  for (int ct = 0; ct < CT; ++ct) {
+    const int sblk = __builtin_amdgcn_readfirstlane(min(ncol[ct] >> 7, (p.N >> 7) - 1));
     if (p.w_layout) {
-      // operand-order storage: per (16-row tile, chunk) one 2 KB block = [half][lane][16 B],
-      // so each of the two loads of a fragment is one contiguous 1 KB wave access
-      const int nb = min(ncol[j] >> 4, (p.N >> 4) - 1);
-      woff[j] = (uint32_t)nb * (uint32_t)KC * 2048u + (uint32_t)lane * 16u;
+      // operand-order storage: per (16-row group, chunk) one 2 KB block = [piece pair][16-byte
+      // piece g][row c][16 B] holding K bytes 64 (pair) + 16 g; lane (j, h) takes pieces
+      // g = 2 (q & 1) + h of pair q >> 1: every load covers two contiguous 512-byte runs
+      const int nb = min((ncol[ct] >> 4) + (j >> 4), (p.N >> 4) - 1);
+      woff[ct] = (uint32_t)nb * (uint32_t)KC * 2048u + (uint32_t)h * 256u + (uint32_t)(j & 15) * 16u;
     } else {
-      // row-major storage: lanes of group g take K bytes [16g, 16g+16) and [64+16g, 64+16g+16)
-      const int n = min(ncol[j] + c, p.N - 1);
-      woff[j] = (uint32_t)n * (uint32_t)K + 16u * g;
+      const int n = min(ncol[ct] + j, p.N - 1);
+      woff[ct] = (uint32_t)n * (uint32_t)K + 16u * h;
     }
-    ws_ptr[j] = QT == 0 ? p.w_scale + ((int64_t)e * (p.N >> 7) + sblk[j]) * KC : nullptr;
+    ws_ptr[ct] = QT == 0 ? p.w_scale + ((int64_t)e * (p.N >> 7) + sblk) * KC : nullptr;
+#ifdef DLB_ABL_L2
+    woff[ct] &= 0x3FFFFu;
+#endif
   }
+#ifdef DLB_ABL_L2
+  wbase = p.w;
+#endif
 
-  f32x4 acc[MT][4];  // [token sub-tile mt][column sub-tile j]
+  f32x16 acc[RT][CT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rt][ct][r] = 0.0f;
 
   // Pipeline: activations move global -> registers -> LDS in stages of SKC chunks, one stage
   // ahead, one barrier per stage; weight fragments sit in a ring of PD chunks, loaded PD-1
-  // chunks ahead of their use; the scale-and-accumulate FMAs of one 16-token step are issued
-  // between the MFMAs of the next step so the matrix pipe does not wait for the VALU.
+  // chunks ahead of their use; the scale-and-accumulate FMAs of one (row tile, column tile)
+  // step are issued between the MFMAs of the next step so the matrix pipe does not wait for
+  // the VALU.
   u32x4 areg[AU];
   float asreg = 0.0f;
-  i32x8 breg[PD][4];
-  // block scales of a wave's sub-tiles: sub-tiles 0,1 and 2,3 share a 128-column block (gate /
-  // up columns; one block for all four in the down GEMM)
+  u32x4 breg[PD][CT][4];
+  // block scales of a wave's tiles: the gate and the up tile lie in different 128-column
+  // blocks, the two tiles of the down GEMM in the same one
   constexpr int NSC = GATED ? 2 : 1;
   float bsreg[PD][NSC];
   const int NS = (KC + SKC - 1) / SKC;
@@ -282,44 +321,37 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     for (int u = 0; u < AU; ++u) *(u32x4*)(dst + (u % RP) * 32 * kARow + (u / RP) * 128) = areg[u];
     if (QT == 0 && aseg < SKC) as_lds[buf][aseg][arow] = asreg;
   };
-  auto load_b = [&](int kc, i32x8 (&b)[4], float (&bs)[NSC]) {
+  auto load_b = [&](int kc, u32x4 (&b)[CT][4], float (&bs)[NSC]) {
     if (kc >= KC) return;
+    const unsigned char* src = wbase + kc * w_kc_stride;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned char* src = wbase + kc * w_kc_stride;
-      const u32x4 lo = *(const u32x4*)(src + woff[j]);
-      const u32x4 hi = *(const u32x4*)(src + w_hi_off + woff[j]);
-      b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
-                   (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    }
+    for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-    for (int q = 0; q < NSC; ++q) bs[q] = QT == 0 ? ws_ptr[2 * q][kc] : 1.0f;
+      for (int q = 0; q < 4; ++q) b[ct][q] = *(const u32x4*)(src + q * w_q_stride + woff[ct]);
+#pragma unroll
+    for (int q = 0; q < NSC; ++q) bs[q] = QT == 0 ? ws_ptr[q][kc] : 1.0f;
   };
 
-  // software pipeline state: products of the previous 16-token step and their scales
-  f32x4 pp[4];
-  float psc[NSC];
+  // software pipeline state: product of the previous step and its scale
+  f32x16 pp;
+  float psc = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) pp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < 16; ++r) pp[r] = 0.0f;
+  // activation fragment of row tile rt, chunk ci of the stage in buffer buf
+  auto read_x = [&](int buf, int ci, int rt, u32x4 (&x)[4], float& as) {
+    const unsigned char* src = a_lds[buf] + (32 * rt + j) * kARow + ci * 128 + 16 * h;
 #pragma unroll
-  for (int q = 0; q < NSC; ++q) psc[q] = 0.0f;
-  // A stage is SKC * MT steps of 16 tokens x one chunk.  Step t issues its 4 MFMAs, each
-  // followed by the FMAs that retire one product of step t - 1 (for the first step of a
-  // stage: the last step of the previous stage); the activation fragment of step t + 1 is
-  // fetched from LDS before the MFMAs of step t so its latency hides behind them.
-  auto read_x = [&](int buf, int ci, int mt, i32x8& x, float& as) {
-    const unsigned char* src = a_lds[buf] + (16 * mt + c) * kARow + ci * 128 + 16 * g;
-    const u32x4 lo = *(const u32x4*)(src);
-    const u32x4 hi = *(const u32x4*)(src + 64);
-    x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
-              (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    as = QT == 0 ? as_lds[buf][ci][16 * mt + c] : 1.0f;
+    for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(src + 32 * q);
+    as = QT == 0 ? as_lds[buf][ci][32 * rt + j] : 1.0f;
   };
+  // A stage is SKC * RT * CT steps.  Step (ci, rt, ct) issues its two MFMAs, each followed by
+  // half of the FMAs that retire the product of the previous step; the activation fragment of
+  // the next row tile is fetched from LDS a row tile (two steps) ahead.
   auto do_stage = [&](auto jtag, int st) {
     constexpr int J = decltype(jtag)::value;  // st % PD
     const int buf = st & 1;
     const int nchunks = min(SKC, KC - st * SKC);  // chunks of this stage that exist (uniform)
-    i32x8 xq[2];
+    u32x4 xq[2][4];
     float asq[2];
     read_x(buf, 0, 0, xq[0], asq[0]);
 #pragma unroll
@@ -332,34 +364,55 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
       if (ci < nchunks) {
         load_b(st * SKC + ci + PD - 1, breg[refill], bsreg[refill]);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const int t = ci * MT + mt;
-          const int pm = (mt == 0) ? MT - 1 : mt - 1;
-          // prefetch the next step's fragment (same stage only)
-          if (mt + 1 < MT) {
-            read_x(buf, ci, mt + 1, xq[(t + 1) & 1], asq[(t + 1) & 1]);
+        for (int rt = 0; rt < RT; ++rt) {
+          const int cur = (ci * RT + rt) & 1;
+          // prefetch the next row tile's fragment (same stage only)
+          if (rt + 1 < RT) {
+            read_x(buf, ci, rt + 1, xq[cur ^ 1], asq[cur ^ 1]);
           } else if (ci + 1 < SKC) {
-            if (ci + 1 < nchunks) read_x(buf, ci + 1, 0, xq[(t + 1) & 1], asq[(t + 1) & 1]);
+            if (ci + 1 < nchunks) read_x(buf, ci + 1, 0, xq[cur ^ 1], asq[cur ^ 1]);
           }
-          if constexpr (QT == 0) {
-            f32x4 pc[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              pc[j] = mfma_fp8(breg[slot][j], xq[t & 1]);
-              acc[pm][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
+          for (int ct = 0; ct < CT; ++ct) {
+            // accumulator that the previous step's product belongs to
+            const int prt = ct == 0 ? (rt == 0 ? RT - 1 : rt - 1) : rt;
+            const int pct = ct == 0 ? CT - 1 : ct - 1;
+            if constexpr (QT == 0) {
+              f32x16 pc;
+#pragma unroll
+              for (int r = 0; r < 16; ++r) pc[r] = 0.0f;
+              pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                  cat8(breg[slot][ct][0], breg[slot][ct][1]), cat8(xq[cur][0], xq[cur][1]), pc, 0, 0,
+                  0, 0, 0, 0);
+#pragma unroll
+              for (int r = 0; r < 8; ++r) acc[prt][pct][r] += pp[r] * psc;
+              // keep the retiring FMAs next to these MFMAs (the optimiser would otherwise sink
+              // them into one long VALU run with nothing to overlap)
+              asm volatile("" : "+v"(acc[prt][pct]));
+              pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                  cat8(breg[slot][ct][2], breg[slot][ct][3]), cat8(xq[cur][2], xq[cur][3]), pc, 0, 0,
+                  0, 0, 0, 0);
+#pragma unroll
+              for (int r = 8; r < 16; ++r) acc[prt][pct][r] += pp[r] * psc;
+              asm volatile("" : "+v"(acc[prt][pct]));
+              pp = pc;
+              psc = asq[cur] * bsreg[slot][GATED ? ct : 0];
+              __builtin_amdgcn_sched_barrier(0);
+            } else {
+              (void)prt;
+              (void)pct;
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                if constexpr (DT == DLB_DTYPE_BF16)
+                  acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                      __builtin_bit_cast(bf16x8, breg[slot][ct][q]),
+                      __builtin_bit_cast(bf16x8, xq[cur][q]), acc[rt][ct], 0, 0, 0);
+                else
+                  acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                      __builtin_bit_cast(f16x8, breg[slot][ct][q]),
+                      __builtin_bit_cast(f16x8, xq[cur][q]), acc[rt][ct], 0, 0, 0);
+              }
             }
-            // keep the retiring FMAs next to these MFMAs (the optimiser would otherwise sink
-            // them into one long VALU run with nothing to overlap)
-            asm volatile("" : "+v"(acc[pm][0]), "+v"(acc[pm][1]), "+v"(acc[pm][2]), "+v"(acc[pm][3]));
-#pragma unroll
-            for (int j = 0; j < 4; ++j) pp[j] = pc[j];
-#pragma unroll
-            for (int q = 0; q < NSC; ++q) psc[q] = asq[t & 1] * bsreg[slot][q];
-          } else {
-            (void)pm;
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              acc[mt][j] = mfma_16bit<DT>(breg[slot][j], xq[t & 1], acc[mt][j]);
           }
         }
       }
@@ -375,94 +428,110 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   store_a(0);
   if (NS > 1) load_a(1);
   __syncthreads();
+  DLB_T();
   for (int st = 0; st < NS; st += PD) {
     do_stage(std::integral_constant<int, 0>{}, st);
     if (PD > 1 && st + 1 < NS) do_stage(std::integral_constant<int, 1 % PD>{}, st + 1);
     if (PD > 2 && st + 2 < NS) do_stage(std::integral_constant<int, 2 % PD>{}, st + 2);
   }
-  // retire the products of the very last step
+  // retire the product of the very last step
+  if constexpr (QT == 0) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
+    for (int r = 0; r < 16; ++r) acc[RT - 1][CT - 1][r] += pp[r] * psc;
+  }
+  DLB_T();
 
-  // ---- epilogues: lane holds token (16*mt + c), columns ncol[j] + 4*g + i
+  // ---- epilogues: lane holds token (32*rt + j), columns ncol[ct] + 8*(r/4) + 4*h + r%4.
+  // A swap between the lane halves turns two 4-column runs into one 8-column run per lane.
   if (GATED && QT == 1) {
     // rounding points of the reference pipeline (fused_moe.py:166,351-352): GEMM result,
     // silu(gate) and the product are each rounded to the activation type
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int64_t orow = row0 + 16 * mt + c;
-      unsigned short* dst = (unsigned short*)p.hq + orow * p.I + nt * 128 + wave * 32 + 4 * g;
+    for (int rt = 0; rt < RT; ++rt) {
+      const int64_t orow = row0 + 32 * rt + j;
+      unsigned short* dst = (unsigned short*)p.hq + orow * p.I + nt * 128 + wave * 32 + 8 * h;
 #pragma unroll
-      for (int jg = 0; jg < 2; ++jg) {
-        float v[4];
+      for (int pr = 0; pr < 2; ++pr) {
+        unsigned int o[2][2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const unsigned int gu = Elem<DT>::pack(acc[mt][jg][i], acc[mt][jg + 2][i]);
-          const float gate = Elem<DT>::lo(gu), up = Elem<DT>::hi(gu);
-          const float sg = Elem<DT>::lo(Elem<DT>::pack(gate / (1.0f + __expf(-gate)), 0.0f));
-          v[i] = sg * up;
+        for (int s = 0; s < 2; ++s) {
+          float v[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int r = 4 * (2 * pr + s) + i;
+            const unsigned int gu = Elem<DT>::pack(acc[rt][0][r], acc[rt][1][r]);
+            const float gate = Elem<DT>::lo(gu), up = Elem<DT>::hi(gu);
+            const float sg = Elem<DT>::lo(Elem<DT>::pack(gate / (1.0f + __expf(-gate)), 0.0f));
+            v[i] = sg * up;
+          }
+          o[s][0] = Elem<DT>::pack(v[0], v[1]);
+          o[s][1] = Elem<DT>::pack(v[2], v[3]);
         }
-        u32x2 o2;
-        o2[0] = Elem<DT>::pack(v[0], v[1]);
-        o2[1] = Elem<DT>::pack(v[2], v[3]);
-        *(u32x2*)(dst + 16 * jg) = o2;
+        swap_halves(o[0][0], o[1][0]);
+        swap_halves(o[0][1], o[1][1]);
+        *(u32x4*)(dst + 16 * pr) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
       }
     }
   } else if (GATED) {
-    float h[MT][2][4];
-    float amax[MT];
+    float hv[RT][16];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      amax[mt] = 0.0f;
+    for (int rt = 0; rt < RT; ++rt) {
+      float amax = 0.0f;
 #pragma unroll
-      for (int jg = 0; jg < 2; ++jg) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float gate = acc[mt][jg][i];
-          const float up = acc[mt][jg + 2][i];
-          const float v = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;  // 1-ulp reciprocal
-          h[mt][jg][i] = v;
-          amax[mt] = fmaxf(amax[mt], fabsf(v));
-        }
+      for (int r = 0; r < 16; ++r) {
+        const float gate = acc[rt][0][r];
+        const float up = acc[rt][1][r];
+        const float v = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;  // 1-ulp reciprocal
+        hv[rt][r] = v;
+        amax = fmaxf(amax, fabsf(v));
       }
-      amax[mt] = fmaxf(amax[mt], __shfl_xor(amax[mt], 16));
-      amax[mt] = fmaxf(amax[mt], __shfl_xor(amax[mt], 32));
-      if (g == 0) red_lds[wave][16 * mt + c] = amax[mt];
+      amax = max_xor32(amax);
+      if (h == 0) red_lds[wave][32 * rt + j] = amax;
     }
     __syncthreads();
     const int scol = nt;  // 128-column group index of the intermediate
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int r = 16 * mt + c;
+    for (int rt = 0; rt < RT; ++rt) {
+      const int r = 32 * rt + j;
       const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
       const float scale = fmaxf(m, kQuantEps) / kFp8Max;
       const float inv = __builtin_amdgcn_rcpf(scale);  // the stored scale stays exact
       const int64_t orow = row0 + r;
+      unsigned int q[4];
 #pragma unroll
-      for (int jg = 0; jg < 2; ++jg) {
-        const unsigned int q = pack4_fp8(h[mt][jg][0] * inv, h[mt][jg][1] * inv,
-                                         h[mt][jg][2] * inv, h[mt][jg][3] * inv);
-        *(unsigned int*)(p.hq + orow * p.I + nt * 128 + wave * 32 + 16 * jg + 4 * g) = q;
-      }
-      if (wave == 0 && g == 0) p.hs[orow * (p.I >> 7) + scol] = scale;
+      for (int s = 0; s < 4; ++s)
+        q[s] = pack4_fp8(hv[rt][4 * s] * inv, hv[rt][4 * s + 1] * inv, hv[rt][4 * s + 2] * inv,
+                         hv[rt][4 * s + 3] * inv);
+      swap_halves(q[0], q[1]);
+      swap_halves(q[2], q[3]);
+      unsigned char* dst = p.hq + orow * p.I + nt * 128 + wave * 32 + 8 * h;
+      *(u32x2*)(dst) = u32x2{q[0], q[1]};
+      *(u32x2*)(dst + 16) = u32x2{q[2], q[3]};
+      if (wave == 0 && h == 0) p.hs[orow * (p.I >> 7) + scol] = scale;
     }
   } else {
     __syncthreads();  // sid_lds visible (also true after the main loop's barriers)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int sid = sid_lds[16 * mt + c];
-      if (sid < p.numel) {
-        const float rw = p.topk_w[sid];
-        unsigned short* orow = (unsigned short*)p.out + (int64_t)sid * p.N;
+    for (int rt = 0; rt < RT; ++rt) {
+      const int sid = sid_lds[32 * rt + j];
+      const bool live = sid < p.numel;
+      const float rw = live ? p.topk_w[sid] : 0.0f;
+      unsigned short* orow = (unsigned short*)p.out + (int64_t)(live ? sid : 0) * p.N;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int n = ncol[j] + 4 * g;
-          if (n < p.N) {
-            u32x2 o2;
-            o2[0] = Elem<DT>::pack(acc[mt][j][0] * rw, acc[mt][j][1] * rw);
-            o2[1] = Elem<DT>::pack(acc[mt][j][2] * rw, acc[mt][j][3] * rw);
-            *(u32x2*)(orow + n) = o2;
+      for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          unsigned int o[2][2];
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const int r = 4 * (2 * pr + s);
+            o[s][0] = Elem<DT>::pack(acc[rt][ct][r] * rw, acc[rt][ct][r + 1] * rw);
+            o[s][1] = Elem<DT>::pack(acc[rt][ct][r + 2] * rw, acc[rt][ct][r + 3] * rw);
           }
+          swap_halves(o[0][0], o[1][0]);
+          swap_halves(o[0][1], o[1][1]);
+          const int n = ncol[ct] + 16 * pr + 8 * h;
+          if (live && n < p.N) *(u32x4*)(orow + n) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
         }
       }
     }
@@ -483,6 +552,7 @@ __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const Mo
     const int logical = xcd * per_xcd + i;
     if (logical < p.grid_real) moe_gemm_fp8_tile<GATED, DT, BM, QT>(p, logical);
     __syncthreads();  // the tile's LDS is reused by the next one
+    DLB_T();
   }
 }
 
@@ -502,7 +572,7 @@ __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const Mo
 // ---------------------------------------------------------------------------------------
 template <bool GATED, int DT, int QT>
 __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const int logical) {
-  constexpr int BM = 128, BN = 256, MT = 4;
+  constexpr int BM = 128, BN = 256;
   constexpr int kWSlot = BN * 128;  // bytes of one weight ring slot
   constexpr int kXSlot = BM * 128;  // bytes of one activation ring slot
   constexpr int kSC = 16;           // chunks of activation scales resident in LDS
@@ -522,13 +592,14 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave id, kept in scalar registers
   const int lane = tid & 63;
-  const int g = lane >> 4;
-  const int c = lane & 15;
+  const int h = lane >> 5;
+  const int j = lane & 31;
   const int rg = w >> 2;  // waves w and w + 4 share a SIMD: give them different row groups
   const int cg = w & 3;
   const int row0 = mb * BM;
   const int K = p.K, KC = p.KC;
 
+  DLB_T();
   if (tid < BM) sid_lds[tid] = p.sorted_ids[row0 + tid];
 
   auto src_row_of = [&](int r) -> int {
@@ -597,57 +668,67 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     }
   };
 
-  // ---- fragment reads: lane (c, g) takes pieces g and g + 4 of row (tile row + c)
-  // Per lane one base pointer per operand and half; slot and tile offsets are a scalar add and
-  // an immediate.  Column sub-tile j starts at tile-local weight row
-  //   gated: (j >> 1) * 128 + cg * 32 + (j & 1) * 16,   down: cg * 64 + j * 16.
-  const int lo_off = c * 128 + (((g) ^ (c >> 1)) & 7) * 16;
-  const int hi_off = c * 128 + (((g + 4) ^ (c >> 1)) & 7) * 16;
-  const int wcg = (GATED ? cg * 32 : cg * 64) * 128;
-  const unsigned char* w_lo = w_lds + wcg + lo_off;
-  const unsigned char* w_hi = w_lds + wcg + hi_off;
-  const unsigned char* x_lo = x_lds + rg * (64 * 128) + lo_off;
-  const unsigned char* x_hi = x_lds + rg * (64 * 128) + hi_off;
-  const float* as_base = &as_lds[0][64 * rg + c];
-  auto read_w = [&](int slot, i32x8 (&b)[4]) {
-    const unsigned char* bl = w_lo + slot * kWSlot;
-    const unsigned char* bh = w_hi + slot * kWSlot;
+  // ---- fragment reads (32x32 MFMA tiles).  Lane (j, h) takes, of row (tile row + j), the
+  // logical 16-byte pieces 2q + h, q = 0..3 (chunk bytes 32 q + 16 h); piece lp of row r sits
+  // in physical piece lp ^ ((r >> 1) & 7), and every tile starts at a multiple of 32 rows, so
+  // the lane's four byte offsets are f0 ^ (32 q), the same for weights and activations.
+  // Column tile ct of the wave starts at tile-local weight row
+  //   gated: ct * 128 + cg * 32,   down: cg * 64 + ct * 32;   row tile rt at 64 rg + 32 rt.
+  const int f0 = j * 128 + (((h ^ (j >> 1)) & 7) << 4);
+  constexpr int kCtStride = GATED ? 128 * 128 : 32 * 128;  // bytes between the wave's column tiles
+  int wf[4], xf[4];  // lane byte offsets inside a ring slot (column tile 0 / row tile 0)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      constexpr int kUp = 128 * 128;  // gated: up rows follow the 128 gate rows
-      const int off = GATED ? (j >> 1) * kUp + (j & 1) * 2048 : j * 2048;
-      const u32x4 lo = *(const u32x4*)(bl + off);
-      const u32x4 hi = *(const u32x4*)(bh + off);
-      b[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
-                   (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  for (int q = 0; q < 4; ++q) {
+    wf[q] = (GATED ? cg * 32 : cg * 64) * 128 + (f0 ^ (q << 5));
+    xf[q] = rg * (64 * 128) + (f0 ^ (q << 5));
+  }
+  const float* as_base = &as_lds[0][64 * rg + j];
+#ifdef DLB_ABL_NOREAD
+  bool first_reads = true;
+#endif
+  auto read_w = [&](int slot, int ct, u32x4 (&b)[4]) {
+#ifdef DLB_ABL_NOREAD
+    if (!first_reads) {
+      asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+      return;
     }
+#endif
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      b[q] = *(const u32x4*)(w_lds + slot * kWSlot + ct * kCtStride + wf[q]);
   };
-  auto read_x = [&](int slot, int kc, int mt, i32x8& x, float& as) {
-    const u32x4 lo = *(const u32x4*)(x_lo + slot * kXSlot + mt * 2048);
-    const u32x4 hi = *(const u32x4*)(x_hi + slot * kXSlot + mt * 2048);
-    x = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
-              (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    as = QT == 0 ? as_base[(kc & (kSC - 1)) * BM + 16 * mt] : 1.0f;
+  auto read_x = [&](int slot, int kc, int rt, u32x4 (&x)[4], float& as) {
+#ifdef DLB_ABL_NOREAD
+    if (!first_reads) {
+      asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(as));
+      return;
+    }
+#endif
+#pragma unroll
+    for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(x_lds + slot * kXSlot + rt * 4096 + xf[q]);
+    as = QT == 0 ? as_base[(kc & (kSC - 1)) * BM + 32 * rt] : 1.0f;
   };
 
   // ---- weight block scales: wave-uniform, one per (128-column block, chunk), read from LDS
-  // (gated: block 0 = gate columns, 1 = up columns; down: the wave's own 128-column block)
+  // (gated: column tile 0 = gate block, 1 = up block; down: the wave's own 128-column block)
   const float* ws_row0 = ws_lds[GATED ? 0 : (cg >> 1)];
   const float* ws_row1 = ws_lds[GATED ? 1 : (cg >> 1)];
 
-  f32x4 acc[MT][4];
+  f32x16 acc[2][2];  // [row tile][column tile]
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  f32x4 pp[4];
-  float psc[2] = {0.0f, 0.0f};
+    for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-  for (int j = 0; j < 4; ++j) pp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int r = 0; r < 16; ++r) acc[rt][ct][r] = 0.0f;
+  f32x16 pp;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) pp[r] = 0.0f;
+  float psc = 0.0f;
 
-  i32x8 b0[4], b1[4];
-  i32x8 xq[2];
-  float asq[2];
+  u32x4 ba[4], bb[4];  // weight fragments of column tile 0 / 1
+  u32x4 x0[4], x1[4];  // activation fragments of row tile 0 / 1
+  float as0 = 1.0f, as1 = 1.0f;
   float wsc[2] = {1.0f, 1.0f}, wsn[2] = {1.0f, 1.0f};
 
   // prologue: scales, chunks 0..2 of the weights and 0..1 of the activations in flight
@@ -665,34 +746,48 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
   }
   __syncthreads();
-  read_w(0, b0);
-  read_x(0, 0, 0, xq[0], asq[0]);
+  DLB_T();
+  read_w(0, 0, ba);
+  read_x(0, 0, 0, x0, as0);
   if (QT == 0) {
     wsc[0] = ws_row0[0];
     wsc[1] = ws_row1[0];
   }
 
-  // one 16-row step: 4 MFMAs, each followed by the FMAs retiring one product of the previous step
-  auto step = [&](const i32x8 (&b)[4], int mt, int cur) {
-    const int pm = (mt == 0) ? MT - 1 : mt - 1;
+  // one (row tile, column tile) step: two MFMAs over the chunk's two 64-byte halves, each
+  // followed by half of the FMAs that retire the previous step's product into `prev`
+  auto step = [&](const u32x4 (&b)[4], const u32x4 (&x)[4], f32x16& own, f32x16& prev, float sc) {
     if constexpr (QT == 0) {
-      f32x4 pc[4];
+      (void)own;
+      f32x16 pc;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        pc[j] = mfma_fp8(b[j], xq[cur]);
-        acc[pm][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
-      }
+      for (int r = 0; r < 16; ++r) pc[r] = 0.0f;
+      pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cat8(b[0], b[1]), cat8(x[0], x[1]), pc, 0,
+                                                           0, 0, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) prev[r] += pp[r] * psc;
       // keep the retiring FMAs inside this step (they would otherwise be sunk past the
       // following steps and run as one block with no MFMA to overlap)
-      asm volatile("" : "+v"(acc[pm][0]), "+v"(acc[pm][1]), "+v"(acc[pm][2]), "+v"(acc[pm][3]));
+      asm volatile("" : "+v"(prev));
+      pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cat8(b[2], b[3]), cat8(x[2], x[3]), pc, 0,
+                                                           0, 0, 0, 0, 0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) pp[j] = pc[j];
-      psc[0] = asq[cur] * wsc[0];
-      psc[1] = asq[cur] * wsc[1];
+      for (int r = 8; r < 16; ++r) prev[r] += pp[r] * psc;
+      asm volatile("" : "+v"(prev));
+      pp = pc;
+      psc = sc;
     } else {
-      (void)pm;
+      (void)prev;
+      (void)sc;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[mt][j] = mfma_16bit<DT>(b[j], xq[cur], acc[mt][j]);
+      for (int q = 0; q < 4; ++q) {
+        if constexpr (DT == DLB_DTYPE_BF16)
+          own = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b[q]),
+                                                        __builtin_bit_cast(bf16x8, x[q]), own, 0, 0, 0);
+        else
+          own = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, b[q]),
+                                                       __builtin_bit_cast(f16x8, x[q]), own, 0, 0, 0);
+      }
     }
   };
   // ring positions as scalars rotated once per chunk (no modulo in the loop): slot of chunk
@@ -700,74 +795,78 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   // the weights of chunk kc + 3 go where chunk kc was)
   int x_cur = 0, x_nxt = 1, x_tgt = 2;
   int w_cur = 0, w_nxt = 1, w_aft = 2;
-  auto rotate = [&]() {
-    wsc[0] = wsn[0];
-    wsc[1] = wsn[1];
-    const int xr = x_cur;
-    x_cur = x_nxt;
-    x_nxt = x_tgt;
-    x_tgt = xr;
-    const int wr = w_cur;
-    w_cur = w_nxt;
-    w_nxt = w_aft;
-    w_aft = wr;
-  };
-  auto do_chunk = [&](const i32x8 (&bc)[4], i32x8 (&bn)[4], int kc) {
+  // Chunk kc, steps in the order (ct 0, rt 0), (ct 0, rt 1), barrier, (ct 1, rt 0), (ct 1, rt 1).
+  // On entry ba = W(kc, ct 0) and x0 = X(kc, rt 0) are in registers; bb and x1 are fetched
+  // during step 0, the next chunk's ba during step 2 and x0 during step 3 (each register set
+  // is free by then and the data landed with the barrier), so every LDS read has at least a
+  // step of MFMAs to hide behind.
+  for (int kc = 0; kc < KC; ++kc) {
     const bool more = kc + 1 < KC;
-    read_x(x_cur, kc, 1, xq[1], asq[1]);
+#ifdef DLB_ABL_NOREAD
+    first_reads = kc == 0;
+#endif
+    read_w(w_cur, 1, bb);
+    read_x(x_cur, kc, 1, x1, as1);
     __builtin_amdgcn_sched_barrier(0);
-    step(bc, 0, 0);
+    step(ba, x0, acc[0][0], acc[1][1], as0 * wsc[0]);
     __builtin_amdgcn_sched_barrier(0);
-    read_x(x_cur, kc, 2, xq[0], asq[0]);
-    __builtin_amdgcn_sched_barrier(0);
-    step(bc, 1, 1);
+    step(ba, x1, acc[1][0], acc[0][0], as1 * wsc[0]);
     __builtin_amdgcn_sched_barrier(0);
     if (more) {
       // chunk kc + 1 has landed once every wave's own loads of it are back
       if (kc + 2 < KC) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);  // W(kc + 2) may still fly
       else __builtin_amdgcn_s_waitcnt(0x0F70);
+#ifndef DLB_ABL_NOBAR
+      __syncthreads();
+#endif
       if (QT == 0 && ((kc + 1) & (kSC - 1)) == 0) {
-        // rare (K > 2048 bytes): next tile of activation scales; every wave is past its reads
-        // of the old tile once it has the step-3 fragment, so fetch that first
-        read_x(x_cur, kc, 3, xq[1], asq[1]);
-        __syncthreads();
+        // rare (K > 2048 bytes): next tile of activation scales; every wave has fetched its
+        // scales of chunk kc before the barrier above
         load_scales(kc + 1);
         __syncthreads();
-      } else {
-        __syncthreads();
-        read_x(x_cur, kc, 3, xq[1], asq[1]);
       }
+#ifndef DLB_ABL_NODMA
       if (kc + 2 < KC) issue_x(kc + 2, x_tgt);
-      read_w(w_nxt, bn);
+#endif
+      read_w(w_nxt, 0, ba);
       if (QT == 0) {
         wsn[0] = ws_row0[(kc + 1) & (kSC - 1)];
         wsn[1] = ws_row1[(kc + 1) & (kSC - 1)];
       }
-    } else {
-      read_x(x_cur, kc, 3, xq[1], asq[1]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    step(bc, 2, 0);
+    step(bb, x0, acc[0][1], acc[1][0], as0 * wsc[1]);
     __builtin_amdgcn_sched_barrier(0);
     // the weights of chunk kc + 3 (least urgent) go out a step after the activations, which
     // spreads the workgroup's requests; still issued after X(kc + 2), as the waits assume
+#ifndef DLB_ABL_NODMA
     if (kc + 3 < KC) issue_w(kc + 3, w_cur);
-    if (more) read_x(x_nxt, kc + 1, 0, xq[0], asq[0]);
+#endif
+    if (more) read_x(x_nxt, kc + 1, 0, x0, as0);
     __builtin_amdgcn_sched_barrier(0);
-    step(bc, 3, 1);
+    step(bb, x1, acc[1][1], acc[0][1], as1 * wsc[1]);
     __builtin_amdgcn_sched_barrier(0);
-    rotate();
-  };
-  for (int kc = 0; kc < KC; kc += 2) {
-    do_chunk(b0, b1, kc);
-    if (kc + 1 < KC) do_chunk(b1, b0, kc + 1);
+    {
+      wsc[0] = wsn[0];
+      wsc[1] = wsn[1];
+      const int xr = x_cur;
+      x_cur = x_nxt;
+      x_nxt = x_tgt;
+      x_tgt = xr;
+      const int wr = w_cur;
+      w_cur = w_nxt;
+      w_nxt = w_aft;
+      w_aft = wr;
+    }
   }
   if constexpr (QT == 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[MT - 1][j] += pp[j] * psc[GATED ? (j >> 1) : 0];
+    for (int r = 0; r < 16; ++r) acc[1][1][r] += pp[r] * psc;
   }
+  DLB_T();
 
-  // ---- epilogues: lane holds slot row (64*rg + 16*mt + c), columns (sub-tile j) + 4*g + i.
+  // ---- epilogues: lane holds slot row (64 rg + 32 rt + j), columns (tile ct) + 8 (r / 4) +
+  // 4 h + r % 4; a swap between the lane halves gives each lane 8 adjacent columns.
   // The output tile is assembled in LDS (the weight ring is free once every wave has left the
   // main loop) and written out as whole rows: 16-byte pieces, a row's pieces on adjacent lanes.
   const int rbase = 64 * rg;
@@ -786,22 +885,28 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     // rounding points of the reference pipeline (fused_moe.py:166,351-352)
     __syncthreads();  // all waves are done with the rings
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      unsigned short* dst = (unsigned short*)stage + (rbase + 16 * mt + c) * 128 + cg * 32 + 4 * g;
+    for (int rt = 0; rt < 2; ++rt) {
+      unsigned short* dst = (unsigned short*)stage + (rbase + 32 * rt + j) * 128 + cg * 32 + 8 * h;
 #pragma unroll
-      for (int jg = 0; jg < 2; ++jg) {
-        float v[4];
+      for (int pr = 0; pr < 2; ++pr) {
+        unsigned int o[2][2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const unsigned int gu = Elem<DT>::pack(acc[mt][jg][i], acc[mt][jg + 2][i]);
-          const float gate = Elem<DT>::lo(gu), up = Elem<DT>::hi(gu);
-          const float sg = Elem<DT>::lo(Elem<DT>::pack(gate / (1.0f + __expf(-gate)), 0.0f));
-          v[i] = sg * up;
+        for (int s = 0; s < 2; ++s) {
+          float v[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int r = 4 * (2 * pr + s) + i;
+            const unsigned int gu = Elem<DT>::pack(acc[rt][0][r], acc[rt][1][r]);
+            const float gate = Elem<DT>::lo(gu), up = Elem<DT>::hi(gu);
+            const float sg = Elem<DT>::lo(Elem<DT>::pack(gate / (1.0f + __expf(-gate)), 0.0f));
+            v[i] = sg * up;
+          }
+          o[s][0] = Elem<DT>::pack(v[0], v[1]);
+          o[s][1] = Elem<DT>::pack(v[2], v[3]);
         }
-        u32x2 o2;
-        o2[0] = Elem<DT>::pack(v[0], v[1]);
-        o2[1] = Elem<DT>::pack(v[2], v[3]);
-        *(u32x2*)(dst + 16 * jg) = o2;
+        swap_halves(o[0][0], o[1][0]);
+        swap_halves(o[0][1], o[1][1]);
+        *(u32x4*)(dst + 16 * pr) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
       }
     }
     __syncthreads();
@@ -809,39 +914,39 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
       return p.hq + ((int64_t)(row0 + r) * p.I + nt * 128) * 2;
     });
   } else if (GATED) {
-    float h[MT][2][4];
+    float hv[2][16];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int rt = 0; rt < 2; ++rt) {
       float amax = 0.0f;
 #pragma unroll
-      for (int jg = 0; jg < 2; ++jg) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float gate = acc[mt][jg][i];
-          const float up = acc[mt][jg + 2][i];
-          const float v = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;  // 1-ulp reciprocal
-          h[mt][jg][i] = v;
-          amax = fmaxf(amax, fabsf(v));
-        }
+      for (int r = 0; r < 16; ++r) {
+        const float gate = acc[rt][0][r];
+        const float up = acc[rt][1][r];
+        const float v = gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate)) * up;  // 1-ulp reciprocal
+        hv[rt][r] = v;
+        amax = fmaxf(amax, fabsf(v));
       }
-      amax = fmaxf(amax, __shfl_xor(amax, 16));
-      amax = fmaxf(amax, __shfl_xor(amax, 32));
-      if (g == 0) red_lds[cg][rbase + 16 * mt + c] = amax;
+      amax = max_xor32(amax);
+      if (h == 0) red_lds[cg][rbase + 32 * rt + j] = amax;
     }
     __syncthreads();  // row maxima visible; all waves are done with the rings
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int r = rbase + 16 * mt + c;
+    for (int rt = 0; rt < 2; ++rt) {
+      const int r = rbase + 32 * rt + j;
       const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
       const float scale = fmaxf(m, kQuantEps) / kFp8Max;
       const float inv = __builtin_amdgcn_rcpf(scale);  // the stored scale stays exact
+      unsigned int q[4];
 #pragma unroll
-      for (int jg = 0; jg < 2; ++jg) {
-        const unsigned int q = pack4_fp8(h[mt][jg][0] * inv, h[mt][jg][1] * inv,
-                                         h[mt][jg][2] * inv, h[mt][jg][3] * inv);
-        *(unsigned int*)(stage + r * 128 + cg * 32 + 16 * jg + 4 * g) = q;
-      }
-      if (cg == 0 && g == 0) p.hs[(int64_t)(row0 + r) * (p.I >> 7) + nt] = scale;
+      for (int s = 0; s < 4; ++s)
+        q[s] = pack4_fp8(hv[rt][4 * s] * inv, hv[rt][4 * s + 1] * inv, hv[rt][4 * s + 2] * inv,
+                         hv[rt][4 * s + 3] * inv);
+      swap_halves(q[0], q[1]);
+      swap_halves(q[2], q[3]);
+      unsigned char* dst = stage + r * 128 + cg * 32 + 8 * h;
+      *(u32x2*)(dst) = u32x2{q[0], q[1]};
+      *(u32x2*)(dst + 16) = u32x2{q[2], q[3]};
+      if (cg == 0 && h == 0) p.hs[(int64_t)(row0 + r) * (p.I >> 7) + nt] = scale;
     }
     __syncthreads();
     flush_rows(128, [&](int r) -> unsigned char* {
@@ -850,17 +955,26 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   } else {
     __syncthreads();  // all waves are done with the rings (and sid_lds is long visible)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int r = rbase + 16 * mt + c;
+    for (int rt = 0; rt < 2; ++rt) {
+      const int r = rbase + 32 * rt + j;
       const int sid = sid_lds[r];
       const float rw = sid < p.numel ? p.topk_w[sid] : 0.0f;
-      unsigned short* dst = (unsigned short*)stage + r * 256 + cg * 64 + 4 * g;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        u32x2 o2;
-        o2[0] = Elem<DT>::pack(acc[mt][j][0] * rw, acc[mt][j][1] * rw);
-        o2[1] = Elem<DT>::pack(acc[mt][j][2] * rw, acc[mt][j][3] * rw);
-        *(u32x2*)(dst + 16 * j) = o2;
+      for (int ct = 0; ct < 2; ++ct) {
+        unsigned short* dst = (unsigned short*)stage + r * 256 + cg * 64 + ct * 32 + 8 * h;
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          unsigned int o[2][2];
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const int a = 4 * (2 * pr + s);
+            o[s][0] = Elem<DT>::pack(acc[rt][ct][a] * rw, acc[rt][ct][a + 1] * rw);
+            o[s][1] = Elem<DT>::pack(acc[rt][ct][a + 2] * rw, acc[rt][ct][a + 3] * rw);
+          }
+          swap_halves(o[0][0], o[1][0]);
+          swap_halves(o[0][1], o[1][1]);
+          *(u32x4*)(dst + 16 * pr) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
+        }
       }
     }
     __syncthreads();
@@ -885,6 +999,7 @@ __global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmPara
     const int logical = xcd * per_xcd + i;
     if (logical < p.grid_real) moe_gemm_wide_tile<GATED, DT, QT>(p, logical);
     __syncthreads();  // the tile's LDS is reused by the next one
+    DLB_T();
   }
 }
 
@@ -917,6 +1032,16 @@ __global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restri
 
 }  // namespace
 }  // namespace dlb
+
+#ifdef DLB_TIMING
+extern "C" int dlb_debug_read(unsigned long long* dst, int* n) {
+  int z = 0;
+  if (hipMemcpyFromSymbol(dst, HIP_SYMBOL(dlb::dbg_t), sizeof(unsigned long long) * 4096) != hipSuccess) return -1;
+  if (hipMemcpyFromSymbol(n, HIP_SYMBOL(dlb::dbg_n), sizeof(int)) != hipSuccess) return -1;
+  if (hipMemcpyToSymbol(HIP_SYMBOL(dlb::dbg_n), &z, sizeof(int)) != hipSuccess) return -1;
+  return 0;
+}
+#endif
 
 extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
                                              int K, int64_t ld_x, int64_t ld_q, int64_t ld_s,
@@ -1052,7 +1177,7 @@ extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const v
                                   num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
   if (!hq || !hs) return DLB_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(hq) & 3u) != 0) return DLB_ERR_UNSUPPORTED;
+  if ((reinterpret_cast<uintptr_t>(hq) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
   p.hq = (unsigned char*)hq;
   p.hs = hs;
   return launch_moe_gemm<true, 0>(p, DLB_DTYPE_BF16, block_m, (hipStream_t)stream);
@@ -1071,7 +1196,7 @@ extern "C" int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void
                                   num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
   if (!out || !topk_weights) return DLB_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(out) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(out)) return DLB_ERR_UNSUPPORTED;
   p.out = out;
   p.topk_w = topk_weights;
   return launch_moe_gemm<false, 0>(p, out_dtype, block_m, (hipStream_t)stream);
@@ -1089,7 +1214,7 @@ extern "C" int dlb_moe_gemm_16bit_gate_up(const void* x, const void* w1,
                                   num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
   if (!act) return DLB_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(act) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(act)) return DLB_ERR_UNSUPPORTED;
   p.hq = (unsigned char*)act;
   return launch_moe_gemm<true, 1>(p, dtype, block_m, (hipStream_t)stream);
 }
@@ -1107,7 +1232,7 @@ extern "C" int dlb_moe_gemm_16bit_down(const void* act, const void* w2,
                                   num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
   if (!out || !topk_weights) return DLB_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(out) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(out)) return DLB_ERR_UNSUPPORTED;
   p.out = out;
   p.topk_w = topk_weights;
   return launch_moe_gemm<false, 1>(p, dtype, block_m, (hipStream_t)stream);
