@@ -144,6 +144,26 @@ __device__ __forceinline__ void dma16_global_to_lds(const void* sbase, unsigned 
                : "memory");
 }
 
+// the 4-byte form: lane l's dword lands at lds_base + 4 * l
+__device__ __forceinline__ void dma4_global_to_lds(const void* gsrc, unsigned int lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :
+               : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base))
+               : "memory");
+}
+
+// the 4-byte form restricted to the lanes of `lane_mask` (a compile-time constant); the other
+// lanes neither read nor write
+template <unsigned long long lane_mask>
+__device__ __forceinline__ void dma4_global_to_lds_masked(const void* gsrc, unsigned int lds_base) {
+  unsigned long long saved;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
+               "global_load_lds_dword %1, off\n\ts_mov_b64 exec, %0"
+               : "=&s"(saved)
+               : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "n"(lane_mask)
+               : "memory");
+}
+
 // ds_read_b64_tr_b16: every lane passes the address of four consecutive 16-bit elements; in
 // each group of 16 lanes the 16 x 4 elements form a 4-row x 16-column block (row j = lanes
 // 4j .. 4j+3 of the group, four columns each) and lane l of the group receives column l,

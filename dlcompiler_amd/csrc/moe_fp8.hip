@@ -148,7 +148,7 @@ __device__ __forceinline__ f32x4 mfma_16bit(const i32x8& a, const i32x8& b, f32x
 // GATED = true : gate_up GEMM (N = 2I), tile = 128 gate cols + the matching 128 up cols,
 //                epilogue silu(gate) * up -> fp8 + per-128 scale, rows kept in sorted order.
 // GATED = false: down GEMM, tile = 256 cols, epilogue * routing weight -> out[slot, n].
-// BM = rows (routing slots) per workgroup = the alignment block of the routing.
+// WL = weight layout (0 row-major, 1 operand order).  64 rows (routing slots) per workgroup.
 //
 // MFMA shape: 32x32x64 (fp8) / 32x32x16 (16 bit).  A wave owns 64 output columns (two 32-column
 // tiles; gated: 32 gate + the matching 32 up columns) x the 64 rows (two 32-row tiles).  Lane
@@ -159,11 +159,22 @@ __device__ __forceinline__ f32x4 mfma_16bit(const i32x8& a, const i32x8& b, f32x
 // an fp8 32x32x64 MFMA (64 cycles) the vector ALU retires the 8 scale-and-accumulate FMAs it
 // owes per MFMA at ~94 % matrix-pipe occupancy, next to the 16x16x128 form (32 cycles, 4 FMAs)
 // only at ~70 %.
+//
+// Data movement, all of it issued by hand so that nothing waits for more than it needs (the
+// compiler's wait-count pass treats a load under a run-time condition as possibly absent and
+// then waits for everything younger too, which defeats a deep prefetch):
+//   * weights: global -> operand registers in units of (chunk, column tile) = 4 x 16 bytes per
+//     lane, a ring of four units, each refilled right after its last use for the chunk after
+//     next (1.5 chunks ahead);
+//   * activations: global -> LDS directly (three chunk slots of 64 x 128 bytes, rows swizzled
+//     by (row >> 1) & 7 in 16-byte pieces), issued two chunks ahead; one barrier per chunk, in
+//     the middle of its MFMAs, publishes the next chunk; the scales of a chunk travel with it
+//     (one 4-byte copy per wave: the activation scales of its 16 staging rows and its own
+//     block scales);
+//   * every wave issues the same number of loads per chunk (chunks past K re-load clamped or
+//     dummy addresses), so the explicit vmcnt waits are compile-time constants.
 #ifndef DLB_MOE_OCC
 #define DLB_MOE_OCC 2
-#endif
-#ifndef DLB_MOE_PD
-#define DLB_MOE_PD 2
 #endif
 
 #ifdef DLB_TIMING
@@ -188,22 +199,49 @@ __device__ __forceinline__ void swap_halves(unsigned int& a, unsigned int& b) {
   b = r[1];
 }
 
-template <bool GATED, int DT, int BM, int QT>
+// one weight unit: the lane's four 16-byte pieces, uniform base + 32-bit lane offset
+template <int WL>
+__device__ __forceinline__ void load_w_unit(u32x4 (&b)[4], unsigned int voff, const unsigned char* sbase) {
+  if constexpr (WL != 0)
+    asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                 "global_load_dwordx4 %1, %4, %5 offset:512\n\t"
+                 "global_load_dwordx4 %2, %4, %5 offset:1024\n\t"
+                 "global_load_dwordx4 %3, %4, %5 offset:1536"
+                 : "=&v"(b[0]), "=&v"(b[1]), "=&v"(b[2]), "=&v"(b[3])
+                 : "v"(voff), "s"(sbase)
+                 : "memory");
+  else
+    asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                 "global_load_dwordx4 %1, %4, %5 offset:32\n\t"
+                 "global_load_dwordx4 %2, %4, %5 offset:64\n\t"
+                 "global_load_dwordx4 %3, %4, %5 offset:96"
+                 : "=&v"(b[0]), "=&v"(b[1]), "=&v"(b[2]), "=&v"(b[3])
+                 : "v"(voff), "s"(sbase)
+                 : "memory");
+}
+// wait until at most N vector-memory operations are outstanding; the unit's registers are
+// tied to the wait so that nothing reads them earlier
+template <int N>
+__device__ __forceinline__ void wait_w_unit(u32x4 (&b)[4]) {
+  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+template <bool GATED, int DT, int QT, int WL>
 __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const int logical) {
-  static_assert(BM == 64, "two 32-row MFMA tiles per workgroup");
-  constexpr int kBM = BM;
-  constexpr int RT = BM / 32;          // 32-token row tiles
-  constexpr int CT = 2;                // 32-column tiles per wave
-  constexpr int SKC = 2;               // 128-byte K chunks per activation stage
-  constexpr int PD = DLB_MOE_PD;       // weight-fragment ring depth (chunks in flight + 1)
-  constexpr int TPR = 256 / BM;        // staging threads per activation row
-  constexpr int AU = SKC * 8 / TPR;    // 16-byte units per staging thread and stage
-  constexpr int kARow = SKC * 128 + 16;  // LDS row pitch of an activation stage (bytes)
-  static_assert(SKC <= TPR, "one staging thread per (row, chunk) loads the scale");
-  __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][kBM * kARow];
-  __shared__ __attribute__((aligned(16))) float as_lds[2][SKC][kBM];
-  __shared__ float red_lds[4][kBM];
-  __shared__ int32_t sid_lds[kBM];
+  constexpr int BM = 64;
+  constexpr int NX = 3;                 // activation chunk slots in LDS
+  constexpr int kXSlot = BM * 128;      // bytes of one slot
+  constexpr int kScWave = 80;           // scale strip of a wave per slot: its 16 x-scales, its w-scales
+  constexpr int kScSlot = 4 * kScWave;
+  constexpr int D = QT == 0 ? 3 : 2;    // direct-to-LDS operations per wave and chunk
+  __shared__ __attribute__((aligned(1024))) unsigned char x_lds[NX * kXSlot];
+  __shared__ __attribute__((aligned(16))) unsigned char sc_lds[NX * kScSlot];
+  __shared__ float red_lds[4][BM];
+  __shared__ int32_t sid_lds[BM];
 
   const int mb = logical % p.num_mblocks;
   const int nt = logical / p.num_mblocks;
@@ -212,40 +250,39 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int h = lane >> 5;
   const int j = lane & 31;
-  const int row0 = mb * kBM;
+  const int row0 = mb * BM;
   const int K = p.K, KC = p.KC;
 
   DLB_T();
-  if (tid < kBM) sid_lds[tid] = p.sorted_ids[row0 + tid];
-  static_assert(AU == SKC * (BM / 32), "staging units per thread");
+  if (tid < BM) sid_lds[tid] = p.sorted_ids[row0 + tid];
 
-  // ---- activation chunk staging.  Data: 8 consecutive lanes fetch one row's 128-byte chunk
-  // (a full cache line per row and instruction), 32 rows per pass, BM / 32 passes per chunk.
-  // Scales: thread (row = tid / TPR, chunk = tid % TPR < SKC) fetches one float per stage.
-  constexpr int RP = BM / 32;            // row passes per chunk
-  const int arow = tid / TPR, aseg = tid % TPR;
-  const int prow = tid >> 3, piece = tid & 7;
-  const unsigned char* a_ptr[RP];
-  const float* as_ptr;
-  {
-    auto src_row_of = [&](int r) -> int64_t {
-      if (GATED) {
-        const int sid = p.sorted_ids[row0 + r];
-        return min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
-      }
-      return row0 + r;
-    };
+  auto src_row_of = [&](int r) -> int64_t {
+    if (GATED) {
+      const int sid = p.sorted_ids[row0 + r];
+      return min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
+    }
+    return row0 + r;
+  };
+  // ---- activation staging: per chunk 8 instructions of 8 rows x 128 bytes, two per wave;
+  // lane -> (row, physical piece), the logical piece it fetches undoes the swizzle
+  const int drow = lane >> 3, dpc = lane & 7;
+  const unsigned char* xsrc[2];
 #pragma unroll
-    for (int k = 0; k < RP; ++k) a_ptr[k] = p.a + src_row_of(32 * k + prow) * K + 16 * piece;
-    as_ptr = QT == 0 ? p.a_scale + src_row_of(arow) * KC : nullptr;
+  for (int i = 0; i < 2; ++i) {
+    const int r = 16 * wave + 8 * i + drow;
+    xsrc[i] = p.a + src_row_of(r) * K + ((dpc ^ ((r >> 1) & 7)) << 4);
   }
+  // scales: one 4-byte copy per wave and chunk with 18 lanes active: lanes 0..15 fetch the
+  // activation scales of the wave's 16 staging rows, lanes 16 / 17 the block scale of the wave's
+  // column tile 0 / 1
+  const float* scsrc = nullptr;
 
   // ---- weight fragments: column tile ct of this wave covers 32 output columns
-  int ncol[CT];  // first column of tile ct in the expert's [N, K] matrix
+  int ncol[2];  // first column of tile ct in the expert's [N, K] matrix
   if (GATED) {
     ncol[0] = nt * 128 + wave * 32;
     ncol[1] = p.I + ncol[0];
@@ -253,19 +290,13 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     ncol[0] = nt * 256 + wave * 64;
     ncol[1] = ncol[0] + 32;
   }
-  // Weight addressing: one wave-uniform base per expert (kept in scalar registers) plus a
-  // 32-bit per-lane byte offset per tile; the block scales of a tile are wave-uniform and come
-  // through scalar loads.
   const unsigned char* wbase = p.w + (int64_t)e * p.N * K;
-  uint32_t woff[CT];
-  const float* ws_ptr[CT];
-  // byte distance between consecutive K chunks / between the four pieces of a lane
-  const int w_kc_stride = p.w_layout ? 2048 : 128;
-  const int w_q_stride = p.w_layout ? 512 : 32;
+  constexpr int kWChunk = WL ? 2048 : 128;  // byte distance between consecutive K chunks
+  uint32_t woff[2];
+  const float* wssrc = nullptr;
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) {
-    const int sblk = __builtin_amdgcn_readfirstlane(min(ncol[ct] >> 7, (p.N >> 7) - 1));
-    if (p.w_layout) {
+  for (int ct = 0; ct < 2; ++ct) {
+    if (WL) {
       // operand-order storage: per (16-row group, chunk) one 2 KB block = [piece pair][16-byte
       // piece g][row c][16 B] holding K bytes 64 (pair) + 16 g; lane (j, h) takes pieces
       // g = 2 (q & 1) + h of pair q >> 1: every load covers two contiguous 512-byte runs
@@ -275,170 +306,184 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
       const int n = min(ncol[ct] + j, p.N - 1);
       woff[ct] = (uint32_t)n * (uint32_t)K + 16u * h;
     }
-    ws_ptr[ct] = QT == 0 ? p.w_scale + ((int64_t)e * (p.N >> 7) + sblk) * KC : nullptr;
-#ifdef DLB_ABL_L2
-    woff[ct] &= 0x3FFFFu;
-#endif
   }
-#ifdef DLB_ABL_L2
-  wbase = p.w;
-#endif
+  if (QT == 0) {
+    const int ct = GATED ? (lane == 17 ? 1 : 0) : 0;
+    const int sblk = min(ncol[ct] >> 7, (p.N >> 7) - 1);
+    scsrc = lane < 16 ? p.a_scale + src_row_of(16 * wave + (lane & 15)) * KC
+                      : p.w_scale + ((int64_t)e * (p.N >> 7) + sblk) * KC;
+  }
 
-  f32x16 acc[RT][CT];
+  const unsigned int x_dst0 = lds_addr(x_lds) + wave * 2048;
+  const unsigned int sc_dst0 = lds_addr(sc_lds) + wave * kScWave;
+  // all direct-to-LDS operations of chunk kc (clamped past the end: the count per chunk is fixed)
+  auto issue_x = [&](int kc, int slot) {
+#ifdef DLB_ABL_NOX
+    if (kc > 2) return;
+#endif
+    const int kcc = min(kc, KC - 1);
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+    for (int i = 0; i < 2; ++i)
+      dma16_global_to_lds(xsrc[i] + kcc * 128, x_dst0 + slot * kXSlot + i * 1024);
+    if constexpr (QT == 0) {
+      dma4_global_to_lds_masked<0x3ffffull>(scsrc + kcc, sc_dst0 + slot * kScSlot);
+    }
+  };
+  // weight unit (kc, ct); past the end every lane re-reads the expert's first 16 bytes
+  auto issue_w = [&](int kc, int ct, u32x4 (&b)[4]) {
+#ifdef DLB_ABL_NOW
+    if (kc > 1) {
+      asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+      return;
+    }
+#endif
+#ifdef DLB_ABL_L2
+    kc &= 1;
+#endif
+    const bool live = kc < KC;
+    const unsigned char* sbase = uniform_ptr(wbase + (live ? kc : 0) * kWChunk);
+    load_w_unit<WL>(b, live ? woff[ct] : 0u, sbase);
+  };
+
+  // ---- fragment reads of the activations: lane (j, h), row tile rt, pieces 2q + h at
+  // physical piece (2q + h) ^ ((j >> 1) & 7): byte offsets f0 ^ (32 q)
+  const int f0 = j * 128 + (((h ^ (j >> 1)) & 7) << 4);
+  int xf[4];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
+  for (int q = 0; q < 4; ++q) xf[q] = f0 ^ (q << 5);
+  // row r's scale sits at (r / 16) * kScWave + (r % 16) * 4 of a slot; rows j and 32 + j are
+  // two waves' strips apart
+  const unsigned char* as_mine = sc_lds + (j >> 4) * kScWave + (j & 15) * 4;
+  const unsigned char* ws_mine = sc_lds + wave * kScWave + 64;
+  auto read_x = [&](int slot, int rt, u32x4 (&x)[4], float& as) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(x_lds + slot * kXSlot + rt * 4096 + xf[q]);
+    as = QT == 0 ? *(const float*)(as_mine + slot * kScSlot + rt * (2 * kScWave)) : 1.0f;
+  };
+
+  f32x16 acc[2][2];  // [row tile][column tile]
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][ct][r] = 0.0f;
-
-  // Pipeline: activations move global -> registers -> LDS in stages of SKC chunks, one stage
-  // ahead, one barrier per stage; weight fragments sit in a ring of PD chunks, loaded PD-1
-  // chunks ahead of their use; the scale-and-accumulate FMAs of one (row tile, column tile)
-  // step are issued between the MFMAs of the next step so the matrix pipe does not wait for
-  // the VALU.
-  u32x4 areg[AU];
-  float asreg = 0.0f;
-  u32x4 breg[PD][CT][4];
-  // block scales of a wave's tiles: the gate and the up tile lie in different 128-column
-  // blocks, the two tiles of the down GEMM in the same one
-  constexpr int NSC = GATED ? 2 : 1;
-  float bsreg[PD][NSC];
-  const int NS = (KC + SKC - 1) / SKC;
-
-  auto load_a = [&](int st) {  // stage st -> registers (chunks past K are clamped, unused)
-    const int kc0 = st * SKC;
-#pragma unroll
-    for (int u = 0; u < AU; ++u) {
-      const int kc = min(kc0 + u / RP, KC - 1);
-      areg[u] = *(const u32x4*)(a_ptr[u % RP] + kc * 128);
-    }
-    if (QT == 0 && aseg < SKC) asreg = as_ptr[min(kc0 + aseg, KC - 1)];
-  };
-  auto store_a = [&](int buf) {
-    unsigned char* dst = a_lds[buf] + prow * kARow + 16 * piece;
-#pragma unroll
-    for (int u = 0; u < AU; ++u) *(u32x4*)(dst + (u % RP) * 32 * kARow + (u / RP) * 128) = areg[u];
-    if (QT == 0 && aseg < SKC) as_lds[buf][aseg][arow] = asreg;
-  };
-  auto load_b = [&](int kc, u32x4 (&b)[CT][4], float (&bs)[NSC]) {
-    if (kc >= KC) return;
-    const unsigned char* src = wbase + kc * w_kc_stride;
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) b[ct][q] = *(const u32x4*)(src + q * w_q_stride + woff[ct]);
-#pragma unroll
-    for (int q = 0; q < NSC; ++q) bs[q] = QT == 0 ? ws_ptr[q][kc] : 1.0f;
-  };
-
-  // software pipeline state: product of the previous step and its scale
   f32x16 pp;
-  float psc = 0.0f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) pp[r] = 0.0f;
-  // activation fragment of row tile rt, chunk ci of the stage in buffer buf
-  auto read_x = [&](int buf, int ci, int rt, u32x4 (&x)[4], float& as) {
-    const unsigned char* src = a_lds[buf] + (32 * rt + j) * kARow + ci * 128 + 16 * h;
+  float psc = 0.0f;
+
+  u32x4 wr[2][2][4];   // weight units [chunk parity][column tile]
+  u32x4 x0[4], x1[4];  // activation fragments of row tile 0 / 1
+  float as0 = 1.0f, as1 = 1.0f;
+
+  // one (row tile, column tile) step: the chunk's MFMAs, each followed by its share of the FMAs
+  // that retire the previous step's product into `prev`
+  auto step = [&](const u32x4 (&b)[4], const u32x4 (&x)[4], f32x16& own, f32x16& prev, float sc) {
+    if constexpr (QT == 0) {
+      (void)own;
+      f32x16 pc;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(src + 32 * q);
-    as = QT == 0 ? as_lds[buf][ci][32 * rt + j] : 1.0f;
-  };
-  // A stage is SKC * RT * CT steps.  Step (ci, rt, ct) issues its two MFMAs, each followed by
-  // half of the FMAs that retire the product of the previous step; the activation fragment of
-  // the next row tile is fetched from LDS a row tile (two steps) ahead.
-  auto do_stage = [&](auto jtag, int st) {
-    constexpr int J = decltype(jtag)::value;  // st % PD
-    const int buf = st & 1;
-    const int nchunks = min(SKC, KC - st * SKC);  // chunks of this stage that exist (uniform)
-    u32x4 xq[2][4];
-    float asq[2];
-    read_x(buf, 0, 0, xq[0], asq[0]);
+      for (int r = 0; r < 16; ++r) pc[r] = 0.0f;
+      pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cat8(b[0], b[1]), cat8(x[0], x[1]), pc, 0,
+                                                           0, 0, 0, 0, 0);
 #pragma unroll
-    for (int ci = 0; ci < SKC; ++ci) {
-      // ring slot of chunk kc = st * SKC + ci is kc % PD, the slot being refilled holds
-      // chunk kc + PD - 1; both are compile-time constants after unrolling
-      constexpr int kBase = (J * SKC) % PD;
-      const int slot = (kBase + ci) % PD;
-      const int refill = (kBase + ci + PD - 1) % PD;
-      if (ci < nchunks) {
-        load_b(st * SKC + ci + PD - 1, breg[refill], bsreg[refill]);
+      for (int r = 0; r < 8; ++r) prev[r] += pp[r] * psc;
+      // keep the retiring FMAs inside this step (the optimiser would otherwise sink them into
+      // one long VALU run with nothing to overlap)
+      asm volatile("" : "+v"(prev));
+      pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cat8(b[2], b[3]), cat8(x[2], x[3]), pc, 0,
+                                                           0, 0, 0, 0, 0);
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          const int cur = (ci * RT + rt) & 1;
-          // prefetch the next row tile's fragment (same stage only)
-          if (rt + 1 < RT) {
-            read_x(buf, ci, rt + 1, xq[cur ^ 1], asq[cur ^ 1]);
-          } else if (ci + 1 < SKC) {
-            if (ci + 1 < nchunks) read_x(buf, ci + 1, 0, xq[cur ^ 1], asq[cur ^ 1]);
-          }
+      for (int r = 8; r < 16; ++r) prev[r] += pp[r] * psc;
+      asm volatile("" : "+v"(prev));
+      pp = pc;
+      psc = sc;
+    } else {
+      (void)prev;
+      (void)sc;
 #pragma unroll
-          for (int ct = 0; ct < CT; ++ct) {
-            // accumulator that the previous step's product belongs to
-            const int prt = ct == 0 ? (rt == 0 ? RT - 1 : rt - 1) : rt;
-            const int pct = ct == 0 ? CT - 1 : ct - 1;
-            if constexpr (QT == 0) {
-              f32x16 pc;
-#pragma unroll
-              for (int r = 0; r < 16; ++r) pc[r] = 0.0f;
-              pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                  cat8(breg[slot][ct][0], breg[slot][ct][1]), cat8(xq[cur][0], xq[cur][1]), pc, 0, 0,
-                  0, 0, 0, 0);
-#pragma unroll
-              for (int r = 0; r < 8; ++r) acc[prt][pct][r] += pp[r] * psc;
-              // keep the retiring FMAs next to these MFMAs (the optimiser would otherwise sink
-              // them into one long VALU run with nothing to overlap)
-              asm volatile("" : "+v"(acc[prt][pct]));
-              pc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                  cat8(breg[slot][ct][2], breg[slot][ct][3]), cat8(xq[cur][2], xq[cur][3]), pc, 0, 0,
-                  0, 0, 0, 0);
-#pragma unroll
-              for (int r = 8; r < 16; ++r) acc[prt][pct][r] += pp[r] * psc;
-              asm volatile("" : "+v"(acc[prt][pct]));
-              pp = pc;
-              psc = asq[cur] * bsreg[slot][GATED ? ct : 0];
-              __builtin_amdgcn_sched_barrier(0);
-            } else {
-              (void)prt;
-              (void)pct;
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                if constexpr (DT == DLB_DTYPE_BF16)
-                  acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                      __builtin_bit_cast(bf16x8, breg[slot][ct][q]),
-                      __builtin_bit_cast(bf16x8, xq[cur][q]), acc[rt][ct], 0, 0, 0);
-                else
-                  acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                      __builtin_bit_cast(f16x8, breg[slot][ct][q]),
-                      __builtin_bit_cast(f16x8, xq[cur][q]), acc[rt][ct], 0, 0, 0);
-              }
-            }
-          }
-        }
+      for (int q = 0; q < 4; ++q) {
+        if constexpr (DT == DLB_DTYPE_BF16)
+          own = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b[q]),
+                                                        __builtin_bit_cast(bf16x8, x[q]), own, 0, 0, 0);
+        else
+          own = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, b[q]),
+                                                       __builtin_bit_cast(f16x8, x[q]), own, 0, 0, 0);
       }
     }
-    if (st + 1 < NS) store_a(buf ^ 1);   // stage st + 1 was loaded into registers a stage ago
-    if (st + 2 < NS) load_a(st + 2);
-    __syncthreads();
   };
 
-  load_a(0);
-#pragma unroll
-  for (int t = 0; t < PD - 1; ++t) load_b(t, breg[t], bsreg[t]);
-  store_a(0);
-  if (NS > 1) load_a(1);
+  // Order of the vector-memory operations of a wave: X(0); then per chunk k = -2, -1, 0, ...
+  //   W(k + 2, ct 0) [4]   X(k + 3) [D]   W(k + 2, ct 1) [4]
+  // (the prologue plays chunks -2 and -1).  Operations complete in order, so "at most n
+  // outstanding" means everything but the youngest n has landed.
+  issue_x(0, 0);
+  issue_w(0, 0, wr[0][0]);
+  issue_x(1, 1);
+  issue_w(0, 1, wr[0][1]);
+  issue_w(1, 0, wr[1][0]);
+  issue_x(2, 2);
+  issue_w(1, 1, wr[1][1]);
+  wait_vm<16 + 2 * D>();  // X(0) landed
   __syncthreads();
   DLB_T();
-  for (int st = 0; st < NS; st += PD) {
-    do_stage(std::integral_constant<int, 0>{}, st);
-    if (PD > 1 && st + 1 < NS) do_stage(std::integral_constant<int, 1 % PD>{}, st + 1);
-    if (PD > 2 && st + 2 < NS) do_stage(std::integral_constant<int, 2 % PD>{}, st + 2);
+  read_x(0, 0, x0, as0);
+
+  int x_cur = 0, x_nxt = 1, x_tgt = 2;  // slots of chunks k, k + 1, k + 2
+  // Chunk k (P = k & 1), steps (ct 0, rt 0), (ct 0, rt 1), barrier, (ct 1, rt 0), (ct 1, rt 1).
+  // On entry x0 = X(k, rt 0) is in registers.
+  auto do_chunk = [&](auto ptag, int k) {
+    constexpr int P = decltype(ptag)::value;
+    float ws0 = 1.0f, ws1 = 1.0f;
+    read_x(x_cur, 1, x1, as1);
+    if constexpr (QT == 0) {
+      ws0 = *(const float*)(ws_mine + x_cur * kScSlot);
+      ws1 = GATED ? *(const float*)(ws_mine + x_cur * kScSlot + 4) : ws0;
+    }
+    wait_w_unit<12 + 2 * D>(wr[P][0]);  // W(k, ct 0) landed
+    __builtin_amdgcn_sched_barrier(0);
+    step(wr[P][0], x0, acc[0][0], acc[1][1], as0 * ws0);
+    __builtin_amdgcn_sched_barrier(0);
+    step(wr[P][0], x1, acc[1][0], acc[0][0], as1 * ws0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_w(k + 2, 0, wr[P][0]);
+    wait_vm<16 + D>();  // this wave's part of X(k + 1) landed
+    __syncthreads();    // X(k + 1) complete; every wave is done reading X(k)
+    issue_x(k + 3, x_cur);
+    wait_w_unit<12 + 2 * D>(wr[P][1]);  // W(k, ct 1) landed
+    __builtin_amdgcn_sched_barrier(0);
+    step(wr[P][1], x0, acc[0][1], acc[1][0], as0 * ws1);
+    __builtin_amdgcn_sched_barrier(0);
+    read_x(x_nxt, 0, x0, as0);
+    __builtin_amdgcn_sched_barrier(0);
+    step(wr[P][1], x1, acc[1][1], acc[0][1], as1 * ws1);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_w(k + 2, 1, wr[P][1]);
+    const int xr = x_cur;
+    x_cur = x_nxt;
+    x_nxt = x_tgt;
+    x_tgt = xr;
+  };
+  for (int k = 0; k < KC; k += 2) {
+    do_chunk(std::integral_constant<int, 0>{}, k);
+    if (k + 1 < KC) do_chunk(std::integral_constant<int, 1>{}, k + 1);
   }
+  // The clamped loads past the end are still in flight and will write the ring's registers:
+  // the wait names those registers, so nothing after it can be given one of them earlier.
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(wr[0][0][0]), "+v"(wr[0][0][1]), "+v"(wr[0][0][2]), "+v"(wr[0][0][3]),
+                 "+v"(wr[0][1][0]), "+v"(wr[0][1][1]), "+v"(wr[0][1][2]), "+v"(wr[0][1][3]),
+                 "+v"(wr[1][0][0]), "+v"(wr[1][0][1]), "+v"(wr[1][0][2]), "+v"(wr[1][0][3]),
+                 "+v"(wr[1][1][0]), "+v"(wr[1][1][1]), "+v"(wr[1][1][2]), "+v"(wr[1][1][3])
+               :
+               : "memory");
   // retire the product of the very last step
   if constexpr (QT == 0) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[RT - 1][CT - 1][r] += pp[r] * psc;
+    for (int r = 0; r < 16; ++r) acc[1][1][r] += pp[r] * psc;
   }
+
   DLB_T();
 
   // ---- epilogues: lane holds token (32*rt + j), columns ncol[ct] + 8*(r/4) + 4*h + r%4.
@@ -447,7 +492,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     // rounding points of the reference pipeline (fused_moe.py:166,351-352): GEMM result,
     // silu(gate) and the product are each rounded to the activation type
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
+    for (int rt = 0; rt < 2; ++rt) {
       const int64_t orow = row0 + 32 * rt + j;
       unsigned short* dst = (unsigned short*)p.hq + orow * p.I + nt * 128 + wave * 32 + 8 * h;
 #pragma unroll
@@ -473,9 +518,9 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
       }
     }
   } else if (GATED) {
-    float hv[RT][16];
+    float hv[2][16];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
+    for (int rt = 0; rt < 2; ++rt) {
       float amax = 0.0f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -491,7 +536,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     __syncthreads();
     const int scol = nt;  // 128-column group index of the intermediate
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
+    for (int rt = 0; rt < 2; ++rt) {
       const int r = 32 * rt + j;
       const float m = fmaxf(fmaxf(red_lds[0][r], red_lds[1][r]), fmaxf(red_lds[2][r], red_lds[3][r]));
       const float scale = fmaxf(m, kQuantEps) / kFp8Max;
@@ -512,13 +557,13 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   } else {
     __syncthreads();  // sid_lds visible (also true after the main loop's barriers)
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
+    for (int rt = 0; rt < 2; ++rt) {
       const int sid = sid_lds[32 * rt + j];
       const bool live = sid < p.numel;
       const float rw = live ? p.topk_w[sid] : 0.0f;
       unsigned short* orow = (unsigned short*)p.out + (int64_t)(live ? sid : 0) * p.N;
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct) {
+      for (int ct = 0; ct < 2; ++ct) {
 #pragma unroll
         for (int pr = 0; pr < 2; ++pr) {
           unsigned int o[2][2];
@@ -544,13 +589,13 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
 // consecutive tiles of it.  With fewer workgroups than tiles (a resident launch, two per CU)
 // every workgroup walks a fixed sequence of tiles; with one workgroup per tile the loop runs
 // once.
-template <bool GATED, int DT, int BM, int QT>
+template <bool GATED, int DT, int QT, int WL>
 __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int per_xcd = (p.grid_real + 7) >> 3;
   for (int i = slot; i < per_xcd; i += slots) {
     const int logical = xcd * per_xcd + i;
-    if (logical < p.grid_real) moe_gemm_fp8_tile<GATED, DT, BM, QT>(p, logical);
+    if (logical < p.grid_real) moe_gemm_fp8_tile<GATED, DT, QT, WL>(p, logical);
     __syncthreads();  // the tile's LDS is reused by the next one
     DLB_T();
   }
@@ -1100,8 +1145,13 @@ int launch_moe_gemm(const MoeGemmParams& p, int dtype, int block_m, hipStream_t 
   // the gated one (+4 %), which therefore keeps one workgroup per tile
   const uint32_t resident = (uint32_t)persistent_workgroups();
   const uint32_t pgrid = (GATED || grid < resident) ? grid : resident;
-#define DLB_LAUNCH_GEMM(DT_) \
-  hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, 64, QT>), dim3(pgrid), dim3(256), 0, s, p)
+#define DLB_LAUNCH_GEMM(DT_)                                                                      \
+  do {                                                                                          \
+    if (p.w_layout)                                                                             \
+      hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, QT, 1>), dim3(pgrid), dim3(256), 0, s, p); \
+    else                                                                                        \
+      hipLaunchKernelGGL((moe_gemm_fp8_kernel<GATED, DT_, QT, 0>), dim3(pgrid), dim3(256), 0, s, p); \
+  } while (0)
   const uint32_t wgrid = grid < resident / 2 ? grid : resident / 2;  // one 8-wave workgroup per CU
 #define DLB_LAUNCH_WIDE(DT_) \
   hipLaunchKernelGGL((moe_gemm_wide_kernel<GATED, DT_, QT>), dim3(wgrid), dim3(512), 0, s, p)
