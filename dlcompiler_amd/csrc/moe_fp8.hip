@@ -241,7 +241,6 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   __shared__ __attribute__((aligned(1024))) unsigned char x_lds[NX * kXSlot];
   __shared__ __attribute__((aligned(16))) unsigned char sc_lds[NX * kScSlot];
   __shared__ float red_lds[4][BM];
-  __shared__ int32_t sid_lds[BM];
 
   const int mb = logical % p.num_mblocks;
   const int nt = logical / p.num_mblocks;
@@ -258,7 +257,16 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   const int K = p.K, KC = p.KC;
 
   DLB_T();
-  if (tid < BM) sid_lds[tid] = p.sorted_ids[row0 + tid];
+  // down GEMM: slot and routing weight of the lane's two rows, fetched now (the loads are older
+  // than everything the main loop issues) and first touched in the epilogue
+  int out_sid[2] = {0, 0};
+  float out_rw[2] = {0.0f, 0.0f};
+  if (!GATED) {
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) out_sid[rt] = p.sorted_ids[row0 + 32 * rt + j];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) out_rw[rt] = out_sid[rt] < p.numel ? p.topk_w[out_sid[rt]] : 0.0f;
+  }
 
   auto src_row_of = [&](int r) -> int64_t {
     if (GATED) {
@@ -355,7 +363,16 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   // two waves' strips apart
   const unsigned char* as_mine = sc_lds + (j >> 4) * kScWave + (j & 15) * 4;
   const unsigned char* ws_mine = sc_lds + wave * kScWave + 64;
+#ifdef DLB_ABL_NOREAD
+  bool abl_started = false;
+#endif
   auto read_x = [&](int slot, int rt, u32x4 (&x)[4], float& as) {
+#ifdef DLB_ABL_NOREAD
+    if (abl_started) {
+      asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(as));
+      return;
+    }
+#endif
 #pragma unroll
     for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(x_lds + slot * kXSlot + rt * 4096 + xf[q]);
     as = QT == 0 ? *(const float*)(as_mine + slot * kScSlot + rt * (2 * kScWave)) : 1.0f;
@@ -449,7 +466,12 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     __builtin_amdgcn_sched_barrier(0);
     issue_w(k + 2, 0, wr[P][0]);
     wait_vm<16 + D>();  // this wave's part of X(k + 1) landed
+#ifdef DLB_ABL_NOREAD
+    abl_started = true;
+#endif
+#ifndef DLB_ABL_NOBAR
     __syncthreads();    // X(k + 1) complete; every wave is done reading X(k)
+#endif
     issue_x(k + 3, x_cur);
     wait_w_unit<12 + 2 * D>(wr[P][1]);  // W(k, ct 1) landed
     __builtin_amdgcn_sched_barrier(0);
@@ -555,12 +577,11 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
       if (wave == 0 && h == 0) p.hs[orow * (p.I >> 7) + scol] = scale;
     }
   } else {
-    __syncthreads();  // sid_lds visible (also true after the main loop's barriers)
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-      const int sid = sid_lds[32 * rt + j];
+      const int sid = out_sid[rt];
       const bool live = sid < p.numel;
-      const float rw = live ? p.topk_w[sid] : 0.0f;
+      const float rw = out_rw[rt];
       unsigned short* orow = (unsigned short*)p.out + (int64_t)(live ? sid : 0) * p.N;
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct) {
@@ -593,6 +614,11 @@ template <bool GATED, int DT, int QT, int WL>
 __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int per_xcd = (p.grid_real + 7) >> 3;
+#ifdef DLB_STAGGER
+  if ((int)blockIdx.x >= DLB_STAGGER_LO && (int)blockIdx.x < DLB_STAGGER_HI) {
+    for (int i = 0; i < DLB_STAGGER; ++i) __builtin_amdgcn_s_sleep(127);
+  }
+#endif
   for (int i = slot; i < per_xcd; i += slots) {
     const int logical = xcd * per_xcd + i;
     if (logical < p.grid_real) moe_gemm_fp8_tile<GATED, DT, QT, WL>(p, logical);
@@ -1141,10 +1167,11 @@ int launch_moe_gemm(const MoeGemmParams& p, int dtype, int block_m, hipStream_t 
     const int64_t a_rows = GATED ? p.num_tokens : (int64_t)p.num_mblocks * 128;
     if (a_rows * p.K >= (int64_t)0xffffffffu) return DLB_ERR_UNSUPPORTED;
   }
-  // measured: walking the tiles with resident workgroups pays for the down GEMM (-5 %), not for
-  // the gated one (+4 %), which therefore keeps one workgroup per tile
+  // measured: one workgroup per tile (the dispatcher hands out tiles as slots free up) beats
+  // resident workgroups walking a fixed share of the tiles, by 10 % for the gated GEMM and 3 %
+  // for the down GEMM: blocks past the routed rows end at once and would unbalance fixed shares
   const uint32_t resident = (uint32_t)persistent_workgroups();
-  const uint32_t pgrid = (GATED || grid < resident) ? grid : resident;
+  const uint32_t pgrid = grid;
 #define DLB_LAUNCH_GEMM(DT_)                                                                      \
   do {                                                                                          \
     if (p.w_layout)                                                                             \
