@@ -1,7 +1,7 @@
 // fp8 (OCP e4m3fn) fused-MoE building blocks for gfx950:
 //   * per-token-group activation quantisation (groups of 128 along K, fp32 scales);
-//   * expert-grouped GEMM over block-aligned routing (64-row blocks, one expert per block) on
-//     the 16x16x128 f8f6f4 MFMA, with the block scales applied per 128-deep K chunk:
+//   * expert-grouped GEMM over block-aligned routing (64- or 128-row blocks, one expert per
+//     block) on the 32x32x64 f8f6f4 MFMA, with the block scales applied per 128-deep K chunk:
 //         acc += mfma(x_q[:, kc], w_q[:, kc]) * x_scale[row, kc] * w_scale[n / 128, kc]
 //     in two flavours -- "gate_up" (A rows gathered by token, SiLU-and-mul and re-quantisation
 //     of the intermediate fused into the epilogue) and "down" (routing weight applied, rows
@@ -15,15 +15,16 @@
 // counterpart there; its nearest precedent is the int8 per-token quantisation and
 // scale-in-epilogue GEMM of python/dlBLAS/dlblas/kernels/w8a8.py:102-106,275-335.
 //
-// The same kernel also runs unquantised bf16/f16 operands (QT = 1): the reference's own
-// fused_moe, with 16x16x32 MFMAs accumulating in place and no scales.
+// The same kernels also run unquantised bf16/f16 operands (QT = 1): the reference's own
+// fused_moe, with 32x32x16 MFMAs accumulating in place and no scales.
 //
 // GEMM mapping.  The MFMA runs "transposed": weight rows are the A operand (M index = output
-// column n), activations the B operand (N index = token row), so a lane's four accumulator
-// registers are four consecutive n of ONE token: the activation scale is a per-lane scalar
-// and the epilogues store 4 adjacent outputs.  Weight fragments go straight from HBM/L2 into
-// operand registers (each wave owns its own n range, so nothing is shared between waves);
-// only the 64 x 128-byte activation chunk is staged through LDS, double-buffered.
+// column n), activations the B operand (N index = token row), so a lane's sixteen accumulator
+// registers of a 32x32 tile are 4 x 4 consecutive n of ONE token: the activation scale is a
+// per-lane scalar and the epilogues store runs of adjacent outputs.  In the 64-row kernel
+// weight fragments go straight from HBM/L2 into operand registers (each wave owns its own n
+// range, so nothing is shared between waves) and only the 64 x 128-byte activation chunk
+// passes through LDS; the 128-row kernel stages both operands in LDS.
 #include <type_traits>
 
 #include "common.h"
@@ -117,32 +118,6 @@ struct MoeGemmParams {
   const float* topk_w;        // [numel]
 };
 
-
-__device__ __forceinline__ f32x4 mfma_fp8(const i32x8& a, const i32x8& b) {
-  const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled opcode
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, z, 0, 0, 0, 0, 0, 0);
-}
-
-template <int DT>
-__device__ __forceinline__ f32x4 mfma_16bit(const i32x8& a, const i32x8& b, f32x4 c) {
-  // one 128-byte chunk = 64 elements = two 16x16x32 steps on the two operand halves
-  typedef __attribute__((ext_vector_type(4))) int i32x4;
-  const i32x4 a0 = {a[0], a[1], a[2], a[3]}, a1 = {a[4], a[5], a[6], a[7]};
-  const i32x4 b0 = {b[0], b[1], b[2], b[3]}, b1 = {b[4], b[5], b[6], b[7]};
-  if constexpr (DT == DLB_DTYPE_BF16) {
-    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a0),
-                                                __builtin_bit_cast(bf16x8, b0), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a1),
-                                                __builtin_bit_cast(bf16x8, b1), c, 0, 0, 0);
-  } else {
-    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a0),
-                                               __builtin_bit_cast(f16x8, b0), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a1),
-                                               __builtin_bit_cast(f16x8, b1), c, 0, 0, 0);
-  }
-  return c;
-}
 
 // QT = 0: fp8 operands with block scales; QT = 1: 16-bit operands of type DT, no scales.
 // GATED = true : gate_up GEMM (N = 2I), tile = 128 gate cols + the matching 128 up cols,
