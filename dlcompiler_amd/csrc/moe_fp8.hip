@@ -217,47 +217,57 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   __shared__ __attribute__((aligned(16))) unsigned char sc_lds[NX * kScSlot];
   __shared__ float red_lds[4][BM];
 
-  const int mb = logical % p.num_mblocks;
-  const int nt = logical / p.num_mblocks;
-  const int e_global = p.expert_ids[mb];
-  const int e = e_global - p.expert_offset;
-  if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
-
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int h = lane >> 5;
   const int j = lane & 31;
+  const int drow = lane >> 3, dpc = lane & 7;
+  const int mb = logical % p.num_mblocks;
+  const int nt = logical / p.num_mblocks;
   const int row0 = mb * BM;
   const int K = p.K, KC = p.KC;
 
+  // The routing slots this lane needs are requested together with the block's expert id, so the
+  // prologue pays one memory round trip for its metadata, not two.  Gated: the rows the lane
+  // stages (two) and the row whose scale it fetches.  Down: the lane's two output rows and
+  // their routing weights (first touched in the epilogue; the loads are older than everything
+  // the main loop issues).
+  int meta_sid[3] = {0, 0, 0};
+  if (GATED) {
+    meta_sid[0] = p.sorted_ids[row0 + 16 * wave + drow];
+    meta_sid[1] = p.sorted_ids[row0 + 16 * wave + 8 + drow];
+    meta_sid[2] = p.sorted_ids[row0 + 16 * wave + (lane & 15)];
+  } else {
+    meta_sid[0] = p.sorted_ids[row0 + j];
+    meta_sid[1] = p.sorted_ids[row0 + 32 + j];
+  }
+  const int e_global = p.expert_ids[mb];
+  const int e = e_global - p.expert_offset;
+  if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
+
   DLB_T();
-  // down GEMM: slot and routing weight of the lane's two rows, fetched now (the loads are older
-  // than everything the main loop issues) and first touched in the epilogue
   int out_sid[2] = {0, 0};
   float out_rw[2] = {0.0f, 0.0f};
   if (!GATED) {
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) out_sid[rt] = p.sorted_ids[row0 + 32 * rt + j];
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) out_rw[rt] = out_sid[rt] < p.numel ? p.topk_w[out_sid[rt]] : 0.0f;
-  }
-
-  auto src_row_of = [&](int r) -> int64_t {
-    if (GATED) {
-      const int sid = p.sorted_ids[row0 + r];
-      return min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
+    for (int rt = 0; rt < 2; ++rt) {
+      out_sid[rt] = meta_sid[rt];
+      out_rw[rt] = out_sid[rt] < p.numel ? p.topk_w[out_sid[rt]] : 0.0f;
     }
+  }
+  // source row of staging row i (gated: the slot's token; pad slots read a valid row)
+  auto src_row_of = [&](int which, int r) -> int64_t {
+    if (GATED) return min(meta_sid[which] / p.topk, p.num_tokens - 1);
     return row0 + r;
   };
   // ---- activation staging: per chunk 8 instructions of 8 rows x 128 bytes, two per wave;
   // lane -> (row, physical piece), the logical piece it fetches undoes the swizzle
-  const int drow = lane >> 3, dpc = lane & 7;
   const unsigned char* xsrc[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int r = 16 * wave + 8 * i + drow;
-    xsrc[i] = p.a + src_row_of(r) * K + ((dpc ^ ((r >> 1) & 7)) << 4);
+    xsrc[i] = p.a + src_row_of(i, r) * K + ((dpc ^ ((r >> 1) & 7)) << 4);
   }
   // scales: one 4-byte copy per wave and chunk with 18 lanes active: lanes 0..15 fetch the
   // activation scales of the wave's 16 staging rows, lanes 16 / 17 the block scale of the wave's
@@ -293,7 +303,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   if (QT == 0) {
     const int ct = GATED ? (lane == 17 ? 1 : 0) : 0;
     const int sblk = min(ncol[ct] >> 7, (p.N >> 7) - 1);
-    scsrc = lane < 16 ? p.a_scale + src_row_of(16 * wave + (lane & 15)) * KC
+    scsrc = lane < 16 ? p.a_scale + src_row_of(2, 16 * wave + (lane & 15)) * KC
                       : p.w_scale + ((int64_t)e * (p.N >> 7) + sblk) * KC;
   }
 
