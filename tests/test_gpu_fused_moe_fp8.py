@@ -51,7 +51,9 @@ def _check(out, ref):
 
 @pytest.mark.parametrize("T,H,I,E,k", [(128, 256, 128, 4, 2), (512, 2048, 1408, 8, 6),
                                        (1, 256, 256, 8, 2), (333, 512, 384, 64, 6),
-                                       (64, 128, 128, 2, 1)])
+                                       (64, 128, 128, 2, 1),
+                                       # K of 4096 / 2304 bytes: more than one 16-chunk window of scales
+                                       (96, 4096, 2304, 4, 2)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_moe_fp8_parity(dev, T, H, I, E, k, dtype, monkeypatch):
     from dlcompiler_amd.kernels import fused_moe as fm
