@@ -155,7 +155,7 @@ struct MoeGemmParams {
 #ifdef DLB_TIMING
 __device__ unsigned long long dbg_t[4096];
 __device__ int dbg_n;
-#define DLB_T() do { if ((blockIdx.x & 511) == 8 && threadIdx.x == 0 && dbg_n < 2040) { dbg_t[2 * dbg_n] = clock64(); dbg_t[2 * dbg_n + 1] = wall_clock64(); ++dbg_n; } } while (0)
+#define DLB_T() do { if ((blockIdx.x == 1032 || blockIdx.x == 2064) && threadIdx.x == 0 && dbg_n < 2040) { dbg_t[2 * dbg_n] = clock64(); dbg_t[2 * dbg_n + 1] = wall_clock64(); ++dbg_n; } } while (0)
 #else
 #define DLB_T() do { } while (0)
 #endif
@@ -599,11 +599,6 @@ template <bool GATED, int DT, int QT, int WL>
 __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const MoeGemmParams p) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int per_xcd = (p.grid_real + 7) >> 3;
-#ifdef DLB_STAGGER
-  if ((int)blockIdx.x >= DLB_STAGGER_LO && (int)blockIdx.x < DLB_STAGGER_HI) {
-    for (int i = 0; i < DLB_STAGGER; ++i) __builtin_amdgcn_s_sleep(127);
-  }
-#endif
   for (int i = slot; i < per_xcd; i += slots) {
     const int logical = xcd * per_xcd + i;
     if (logical < p.grid_real) moe_gemm_fp8_tile<GATED, DT, QT, WL>(p, logical);
