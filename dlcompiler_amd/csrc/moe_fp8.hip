@@ -525,6 +525,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
       }
     }
   } else if (GATED) {
+    constexpr int kGatedPitch = 128 + 16;  // staging row pitch of the fp8 output tile
     float hv[2][16];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
@@ -556,18 +557,33 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
                          hv[rt][4 * s + 3] * inv);
       swap_halves(q[0], q[1]);
       swap_halves(q[2], q[3]);
-      unsigned char* dst = p.hq + orow * p.I + nt * 128 + wave * 32 + 8 * h;
+      // staged in the activation slots (free: the barrier above came after every wave's main
+      // loop) so that the tile leaves as whole 128-byte rows
+      unsigned char* dst = x_lds + r * kGatedPitch + wave * 32 + 8 * h;
       *(u32x2*)(dst) = u32x2{q[0], q[1]};
       *(u32x2*)(dst + 16) = u32x2{q[2], q[3]};
       if (wave == 0 && h == 0) p.hs[orow * (p.I >> 7) + scol] = scale;
     }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {  // 64 rows x 8 pieces of 16 bytes, adjacent lanes on one row
+      const int r = (tid >> 3) + 32 * i, pc = tid & 7;
+      *(u32x4*)(p.hq + (int64_t)(row0 + r) * p.I + nt * 128 + 16 * pc) =
+          *(const u32x4*)(x_lds + r * kGatedPitch + 16 * pc);
+    }
   } else {
+    // The 64 x 256 output tile goes out through LDS, one 32-row half at a time (the activation
+    // slots are free once every wave has left the main loop): a lane holds 16-byte runs of 32
+    // different rows, the staged copy writes whole 512-byte rows with adjacent lanes on adjacent
+    // 16-byte pieces.
+    constexpr int kPitch = 512 + 16;  // staging row pitch: rows 16 bytes apart in the banks
+    static_assert(32 * kPitch <= NX * kXSlot, "output staging fits the activation slots");
+    unsigned char* stage = x_lds;
+    const int ncols = min(256, p.N - nt * 256);  // multiple of 128
+    __syncthreads();  // every wave is done reading the activation slots
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-      const int sid = out_sid[rt];
-      const bool live = sid < p.numel;
       const float rw = out_rw[rt];
-      unsigned short* orow = (unsigned short*)p.out + (int64_t)(live ? sid : 0) * p.N;
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct) {
 #pragma unroll
@@ -581,10 +597,22 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
           }
           swap_halves(o[0][0], o[1][0]);
           swap_halves(o[0][1], o[1][1]);
-          const int n = ncol[ct] + 16 * pr + 8 * h;
-          if (live && n < p.N) *(u32x4*)(orow + n) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
+          *(u32x4*)(stage + j * kPitch + (wave * 64 + ct * 32 + 16 * pr + 8 * h) * 2) =
+              u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
         }
       }
+      __syncthreads();
+      // 32 rows x 32 pieces; thread t takes piece t % 32 of rows t / 32 + 8 i.  Row r's slot id
+      // sits in lane r of every wave.
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = (tid >> 5) + 8 * i, pc = tid & 31;
+        const int sid = __shfl(out_sid[rt], r);
+        if (sid < p.numel && 8 * pc < ncols)
+          *(u32x4*)((unsigned short*)p.out + (int64_t)sid * p.N + nt * 256 + 8 * pc) =
+              *(const u32x4*)(stage + r * kPitch + 16 * pc);
+      }
+      if (rt == 0) __syncthreads();  // the second half reuses the staging rows
     }
   }
 }
@@ -1234,7 +1262,7 @@ extern "C" int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const v
                                   num_local_experts, w_layout);
   if (st != DLB_OK || num_mblocks == 0) return st;
   if (!hq || !hs) return DLB_ERR_BAD_ARG;
-  if ((reinterpret_cast<uintptr_t>(hq) & 7u) != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(hq)) return DLB_ERR_UNSUPPORTED;
   p.hq = (unsigned char*)hq;
   p.hs = hs;
   return launch_moe_gemm<true, 0>(p, DLB_DTYPE_BF16, block_m, (hipStream_t)stream);

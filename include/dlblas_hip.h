@@ -196,9 +196,8 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
  * block_m selects the kernel: 64 = four-wave tiles of 64 rows, weights streamed straight into
  * operand registers (fastest with w_layout 1); 128 = eight-wave tiles of 128 rows x 256
  * columns with both operands staged by direct-to-LDS loads (reads row-major weights, w_layout
- * 0, at full efficiency).  Outputs are stored 8 or 16 bytes at a time: hq must be 8-byte
- * aligned (16 with block_m 128), out and the 16-bit act 16-byte aligned; other alignments
- * return DLB_ERR_UNSUPPORTED.
+ * 0, at full efficiency).  Outputs are stored 16 bytes at a time: hq, out and the 16-bit act
+ * must be 16-byte aligned; other alignments return DLB_ERR_UNSUPPORTED.
  * w_layout selects how the fp8 weight bytes of both GEMMs are stored:
  *   0  row-major [E, N, K] (the reference's w1/w2 layout);
  *   1  MFMA-operand order, a one-time re-arrangement done when the weights are loaded: for
