@@ -662,12 +662,6 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   __shared__ float red_lds[4][BM];
   __shared__ int32_t sid_lds[BM];
 
-  const int mb = logical % p.num_mblocks;
-  const int nt = logical / p.num_mblocks;
-  const int e_global = p.expert_ids[mb];
-  const int e = e_global - p.expert_offset;
-  if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
-
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave id, kept in scalar registers
   const int lane = tid & 63;
@@ -675,22 +669,35 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   const int j = lane & 31;
   const int rg = w >> 2;  // waves w and w + 4 share a SIMD: give them different row groups
   const int cg = w & 3;
+  const int drow = lane >> 3, dpc = lane & 7;
+  const int mb = logical % p.num_mblocks;
+  const int nt = logical / p.num_mblocks;
   const int row0 = mb * BM;
   const int K = p.K, KC = p.KC;
 
-  DLB_T();
-  if (tid < BM) sid_lds[tid] = p.sorted_ids[row0 + tid];
+  // the routing slots this thread needs (row tid % 128 for the slot list and the scales, the two
+  // rows it stages) are requested together with the block's expert id: one round trip, not two
+  const int sid_mine = p.sorted_ids[row0 + (tid & (BM - 1))];
+  int sid_x[2] = {0, 0};
+  if (GATED) {
+    sid_x[0] = p.sorted_ids[row0 + 16 * w + drow];
+    sid_x[1] = p.sorted_ids[row0 + 16 * w + 8 + drow];
+  }
+  const int e_global = p.expert_ids[mb];
+  const int e = e_global - p.expert_offset;
+  if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
 
-  auto src_row_of = [&](int r) -> int {
-    if (GATED) {
-      const int sid = p.sorted_ids[row0 + r];
-      return min(sid / p.topk, p.num_tokens - 1);  // pad slots read a valid row
-    }
+  DLB_T();
+  if (tid < BM) sid_lds[tid] = sid_mine;
+
+  // source row of tile row r whose routing slot is sid (gated: the slot's token; pad slots read
+  // a valid row)
+  auto src_row_of = [&](int sid, int r) -> int {
+    if (GATED) return min(sid / p.topk, p.num_tokens - 1);
     return row0 + r;
   };
 
   // ---- direct-to-LDS staging: instruction = 8 rows x 128 bytes, lane -> (row, physical piece)
-  const int drow = lane >> 3, dpc = lane & 7;
   uint32_t w_voff[4], x_voff[2];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -710,7 +717,7 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   for (int q = 0; q < 2; ++q) {
     const int r = 16 * w + 8 * q + drow;
     const int lc = dpc ^ ((r >> 1) & 7);
-    x_voff[q] = (uint32_t)src_row_of(r) * (uint32_t)K + (uint32_t)lc * 16u;
+    x_voff[q] = (uint32_t)src_row_of(sid_x[q], r) * (uint32_t)K + (uint32_t)lc * 16u;
   }
   const unsigned char* wbase = p.w + (int64_t)e * p.N * K;
   const int w_kc_stride = p.w_layout ? 2048 : 128;
@@ -734,7 +741,7 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   auto load_scales = [&](int kc0) {
     if (QT != 0) return;
     const int r = tid & (BM - 1), kq = tid >> 7;
-    const float* sp = p.a_scale + (int64_t)src_row_of(r) * KC;
+    const float* sp = p.a_scale + (int64_t)src_row_of(sid_mine, r) * KC;
 #pragma unroll
     for (int i = 0; i < kSC / 4; ++i) {
       const int kk = kq * (kSC / 4) + i;
@@ -810,19 +817,20 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   float as0 = 1.0f, as1 = 1.0f;
   float wsc[2] = {1.0f, 1.0f}, wsn[2] = {1.0f, 1.0f};
 
-  // prologue: scales, chunks 0..2 of the weights and 0..1 of the activations in flight
-  load_scales(0);
+  // prologue: chunks 0..2 of the weights and 0..1 of the activations in flight, then the scales
+  // (plain loads: issued after the copies so that they do not hold the copies back; the wait the
+  // compiler puts before their LDS stores also covers every copy, which is older)
   issue_x(0, 0);
   issue_w(0, 0);
   if (KC > 1) {
     issue_x(1, 1);
     issue_w(1, 1);
   }
-  if (KC > 2) {
-    issue_w(2, 2);
-    __builtin_amdgcn_s_waitcnt(0x0F70 | 10);  // vmcnt(10): chunk 0 landed, 10 newer loads may fly
-  } else {
-    __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
+  if (KC > 2) issue_w(2, 2);
+  load_scales(0);
+  if (QT != 0) {
+    if (KC > 2) __builtin_amdgcn_s_waitcnt(0x0F70 | 10);  // vmcnt(10): chunk 0 landed
+    else __builtin_amdgcn_s_waitcnt(0x0F70);              // vmcnt(0)
   }
   __syncthreads();
   DLB_T();
