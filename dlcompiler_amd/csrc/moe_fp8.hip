@@ -497,11 +497,14 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   // A swap between the lane halves turns two 4-column runs into one 8-column run per lane.
   if (GATED && QT == 1) {
     // rounding points of the reference pipeline (fused_moe.py:166,351-352): GEMM result,
-    // silu(gate) and the product are each rounded to the activation type
+    // silu(gate) and the product are each rounded to the activation type.  The 64 x 128 tile
+    // is staged in the activation slots and leaves as whole 256-byte rows.
+    constexpr int kActPitch = 256 + 16;
+    static_assert(BM * kActPitch <= NX * kXSlot, "output staging fits the activation slots");
+    __syncthreads();  // every wave is done reading the activation slots
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-      const int64_t orow = row0 + 32 * rt + j;
-      unsigned short* dst = (unsigned short*)p.hq + orow * p.I + nt * 128 + wave * 32 + 8 * h;
+      unsigned short* dst = (unsigned short*)(x_lds + (32 * rt + j) * kActPitch) + wave * 32 + 8 * h;
 #pragma unroll
       for (int pr = 0; pr < 2; ++pr) {
         unsigned int o[2][2];
@@ -523,6 +526,13 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
         swap_halves(o[0][1], o[1][1]);
         *(u32x4*)(dst + 16 * pr) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
       }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // 64 rows x 16 pieces of 16 bytes, adjacent lanes on one row
+      const int r = (tid >> 4) + 16 * i, pc = tid & 15;
+      *(u32x4*)((unsigned short*)p.hq + (int64_t)(row0 + r) * p.I + nt * 128 + 8 * pc) =
+          *(const u32x4*)(x_lds + r * kActPitch + 16 * pc);
     }
   } else if (GATED) {
     constexpr int kGatedPitch = 128 + 16;  // staging row pitch of the fp8 output tile
