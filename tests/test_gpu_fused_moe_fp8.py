@@ -174,3 +174,32 @@ def test_config5_full(dev):
     pick = torch.arange(0, T, 37)
     ref = ofm.fused_moe_fp8(x[pick], w1q, w1s, w2q, w2s, tw[pick], ids[pick])
     _check(out[pick], ref)
+
+
+@pytest.mark.parametrize("block", [64, 128])
+def test_fused_moe_fp8_repeats_bit_identically(dev, block, monkeypatch):
+    """Config-size run, repeated: the kernels issue their loads by hand with explicit waits, so a
+    missing wait would show as run-to-run differences on a busy chip."""
+    from dlcompiler_amd.kernels import fused_moe as fm
+
+    T, H, I, E, k = 4096, 2048, 1408, 64, 6
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn((T, H), generator=g).bfloat16().to(dev)
+    w1q = (torch.randn((E, 2 * I, H), generator=g) * 0.5).to(torch.float8_e4m3fn).to(dev)
+    w2q = (torch.randn((E, H, I), generator=g) * 0.5).to(torch.float8_e4m3fn).to(dev)
+    w1s = (torch.rand((E, 2 * I // 128, H // 128), generator=g) * 0.02 + 0.01).to(dev)
+    w2s = (torch.rand((E, H // 128, I // 128), generator=g) * 0.02 + 0.01).to(dev)
+    tw, ids = torch.topk(torch.softmax(torch.randn((T, E), generator=g), -1), k)
+    tw, ids = tw.to(dev), ids.int().to(dev)
+    monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+    for shuffled in (False, True):
+        a = fm.shuffle_moe_weight_fp8(w1q) if shuffled else w1q
+        b = fm.shuffle_moe_weight_fp8(w2q) if shuffled else w2q
+        first = fm.fused_moe_fp8(x, a, w1s, b, w2s, tw, ids, k, weights_shuffled=shuffled).clone()
+        assert torch.isfinite(first.float()).all()
+        for _ in range(8):
+            again = fm.fused_moe_fp8(x, a, w1s, b, w2s, tw, ids, k, weights_shuffled=shuffled)
+            assert torch.equal(again, first)
+    # both weight layouts hold the same numbers: same result
+    plain = fm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids, k, weights_shuffled=False)
+    assert torch.equal(plain, first)
