@@ -87,3 +87,48 @@ def test_decode_sweep(dev, seed):
                         torch.arange(B, device=dev), torch.ones(B, dtype=torch.int64, device=dev),
                         kl.to(dev), 1, window_size=window, logit_softcapping=softcap)
     _close(o.cpu(), oa.paged_decode(q, kc, vc, table, kl, window=window, softcap=softcap))
+
+
+def test_config_size_attention_repeats_bit_identically(dev):
+    """Config-size prefill and paged decode, repeated: both kernels copy K/V into LDS with
+    hand-issued loads and explicit waits; a missing wait would show as run-to-run differences."""
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    g = torch.Generator().manual_seed(21)
+    Hq, Hkv, D, page = 32, 8, 128, 64
+    lens = torch.randint(512, 4097, (8,), generator=g, dtype=torch.int32)
+    start = (torch.cumsum(lens, 0, dtype=torch.int32) - lens).to(dev)
+    total = int(lens.sum())
+    q = torch.randn((total, Hq, D), generator=g).bfloat16().to(dev)
+    k = torch.randn((total, Hkv, D), generator=g).bfloat16().to(dev)
+    v = torch.randn((total, Hkv, D), generator=g).bfloat16().to(dev)
+    o = torch.empty_like(q)
+    lens_d = lens.to(dev)
+    context_attention_fwd(q, k, v, o, start, lens_d, int(lens.max()))
+    first = o.clone()
+    assert torch.isfinite(first.float()).all()
+    for _ in range(5):
+        o.zero_()
+        context_attention_fwd(q, k, v, o, start, lens_d, int(lens.max()))
+        assert torch.equal(o, first)
+
+    B = 64
+    ctx = torch.randint(512, 8193, (B,), generator=g, dtype=torch.int32)
+    pages_per = 8192 // page
+    npages = B * pages_per
+    kc = torch.randn((npages, page, Hkv, D), generator=g).bfloat16().to(dev)
+    vc = torch.randn((npages, page, Hkv, D), generator=g).bfloat16().to(dev)
+    bt = torch.randperm(npages, generator=g).to(torch.int32).view(B, pages_per).to(dev)
+    qd = torch.randn((B, Hq, D), generator=g).bfloat16().to(dev)
+    od = torch.empty_like(qd)
+    qsl = torch.arange(B, dtype=torch.int32).to(dev)
+    qlen = torch.ones(B, dtype=torch.int32).to(dev)
+    ctx_d = ctx.to(dev)
+    paged_attention_fwd(qd, kc, vc, od, bt, qsl, qlen, ctx_d, 1)
+    firstd = od.clone()
+    assert torch.isfinite(firstd.float()).all()
+    for _ in range(5):
+        od.zero_()
+        paged_attention_fwd(qd, kc, vc, od, bt, qsl, qlen, ctx_d, 1)
+        assert torch.equal(od, firstd)
