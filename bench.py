@@ -65,28 +65,23 @@ class Timer:
         return sum(a.elapsed_time(b) for a, b in self.pairs) / max(len(self.pairs), 1)
 
 
-def _time_steps(step, steps, warmup, per_step_events=True):
-    """step(i) launches one step; returns (ms_per_step over the whole region, per-step mean).
-
-    With ``per_step_events`` every step inside the timed region is also bracketed by its own
-    event pair (the per-launch duration of a single-kernel workload).  Workloads whose dominant
-    kernel is timed separately pass False: two event records per step cost about 10 us of host
-    time, a quarter of the shortest workload's step, and would only dilute the region."""
+def _time_steps(step, steps, warmup):
+    """step(i) launches one step; returns (ms_per_step, ms_per_step): the K steps are bracketed
+    by one event before and one after on the launch stream, and nothing else is recorded inside
+    the region (an event pair around every step costs about 10 us of host time and 7 us of GPU
+    time per step -- a quarter of the shortest workload).  For a single-kernel workload the
+    region divided by K is also that kernel's average launch duration, launch gaps included."""
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     t_all = Timer()
-    t_each = Timer()
     ev = t_all.start()
     for i in range(steps):
-        if per_step_events:
-            e = t_each.start()
         step(i)
-        if per_step_events:
-            t_each.stop(e)
     t_all.stop(ev)
     torch.cuda.synchronize()
-    return t_all.mean_ms() / steps, (t_each.mean_ms() if per_step_events else None)
+    ms = t_all.mean_ms() / steps
+    return ms, ms
 
 
 def _traffic(name):
@@ -180,7 +175,7 @@ def wl_gating(dev, steps, warmup, cpu):
     _, _, npad = step(0)
     l_pad = int(npad.item())
     bytes_ = (T * E * 4 + T * K * 4 * 2 + T * K * 4 + 4 * l_pad + 4 * l_pad // BLK + E * 4 + 4)
-    ms, _ = _time_steps(step, steps, warmup, per_step_events=False)
+    ms, _ = _time_steps(step, steps, warmup)
 
     # the same two calls replayed from a HIP graph (no Python / launch latency in between)
     graph_ms = _graph_replay_ms(lambda: step(0), steps, warmup, "gating")
@@ -350,7 +345,7 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
     gate_up_flops = 2 * T * K * H * 2 * I
 
     ms, _ = _time_steps(lambda i: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled),
-                        steps, warmup, per_step_events=False)
+                        steps, warmup)
 
     graph_ms = _graph_replay_ms(
         lambda: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled), steps, warmup, "moe")
