@@ -189,6 +189,13 @@ __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// tokens per workgroup of the fused router + chunk-histogram kernel = tokens per alignment chunk
+// when the two run as one pipeline
+constexpr int kRouteChunkTokens = 128;  // 64 and 256 measured slower at 16384 tokens
+int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
+                              int K, int64_t ld_logits, int renormalize, int32_t* chunk_counts,
+                              hipStream_t s);
+
 // status of the launch just issued on this thread
 inline int launch_status() { return hipGetLastError() == hipSuccess ? DLB_OK : DLB_ERR_LAUNCH; }
 

@@ -187,9 +187,9 @@ constexpr int kFusedChunks = 256;
 
 __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
     const int32_t* __restrict__ ids, int64_t numel, int E, int block,
-    const int32_t* __restrict__ chunk_counts, int chunks, int32_t* __restrict__ sorted_ids,
-    int64_t sorted_cap, int32_t* __restrict__ expert_ids, int64_t expert_ids_cap,
-    int32_t* __restrict__ counts, int32_t* __restrict__ num_post_pad) {
+    const int32_t* __restrict__ chunk_counts, int chunks, int chunk_ids,
+    int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_ids_cap, int32_t* __restrict__ counts, int32_t* __restrict__ num_post_pad) {
   __shared__ int32_t cursor[kMaxE];            // next free slot per expert for this chunk
   __shared__ int32_t wave_cnt[kWaves][kMaxE];  // per-tile, per-wave counts
   __shared__ int32_t total_s[kMaxE];
@@ -271,8 +271,8 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   }
   __syncthreads();
 
-  const int64_t begin = (int64_t)me * kChunk;
-  const int64_t end = begin + kChunk < numel ? begin + kChunk : numel;
+  const int64_t begin = (int64_t)me * chunk_ids;  // chunk_ids flat ids per chunk (kChunk by default)
+  const int64_t end = begin + chunk_ids < numel ? begin + chunk_ids : numel;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   for (int64_t tile = begin; tile < end; tile += kThreads) {  // uniform trip count
     const int64_t i = tile + tid;
@@ -343,8 +343,8 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
   if (chunks <= kFusedChunks) {
     // (with numel = 0 the single chunk is empty: the extra workgroup still writes pads, tails and totals)
     hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s,
-                       topk_ids, numel, E, block, chunk_counts, (int)chunks, sorted_ids, sorted_cap,
-                       expert_ids, expert_ids_cap, counts, num_post_pad);
+                       topk_ids, numel, E, block, chunk_counts, (int)chunks, kChunk, sorted_ids,
+                       sorted_cap, expert_ids, expert_ids_cap, counts, num_post_pad);
     return launch_status();
   }
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, chunk_counts, chunks, E, block,
@@ -353,5 +353,52 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
   if (numel > 0)
     hipLaunchKernelGGL(align_place_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
                        numel, E, chunk_counts, sorted_ids);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Router and alignment as one pipeline of two launches: the router kernel also writes the
+// per-chunk expert counts (a chunk = the K routing slots of kRouteChunkTokens consecutive
+// tokens), so the alignment's own counting pass over the ids is not needed.
+// ---------------------------------------------------------------------------------------
+extern "C" size_t dlb_moe_topk_softmax_align_ws_bytes(int64_t T, int E) {
+  if (T < 0 || E < 1) return 0;
+  const int64_t chunks = T > 0 ? dlb::ceil_div(T, dlb::kRouteChunkTokens) : 1;
+  return (size_t)chunks * (size_t)E * sizeof(int32_t);
+}
+
+extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t* ids,
+                                              int64_t T, int E, int K, int64_t ld_logits,
+                                              int renormalize, int block, int32_t* sorted_ids,
+                                              int64_t sorted_cap, int32_t* expert_ids,
+                                              int64_t expert_ids_cap, int32_t* counts,
+                                              int32_t* num_post_pad, void* ws, size_t ws_bytes,
+                                              void* stream) {
+  using namespace dlb;
+  if (T < 0 || E < 1 || K < 1 || K > E || ld_logits < E || block < 1) return DLB_ERR_BAD_ARG;
+  if (K > 16 || E > kMaxE) return DLB_ERR_UNSUPPORTED;
+  const int64_t numel = T * K;
+  if (numel + (int64_t)E * block >= (int64_t)0x7fffffff) return DLB_ERR_UNSUPPORTED;
+  const int64_t chunks = T > 0 ? ceil_div(T, kRouteChunkTokens) : 1;
+  // larger inputs take the two separate entry points (their scan runs as its own launch)
+  if (chunks > kFusedChunks) return DLB_ERR_UNSUPPORTED;
+  if (!sorted_ids || !expert_ids || !num_post_pad || (T > 0 && (!logits || !weights || !ids)))
+    return DLB_ERR_BAD_ARG;
+  if (sorted_cap < numel + (int64_t)E * (block - 1)) return DLB_ERR_BAD_ARG;
+  if (expert_ids_cap < ceil_div(sorted_cap, block)) return DLB_ERR_BAD_ARG;
+  if (!ws || ws_bytes < dlb_moe_topk_softmax_align_ws_bytes(T, E)) return DLB_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  int32_t* chunk_counts = (int32_t*)ws;
+  if (T > 0) {
+    const int st = launch_topk_softmax_count(logits, weights, ids, T, E, K, ld_logits, renormalize,
+                                             chunk_counts, s);
+    if (st != DLB_OK) return st;
+  } else {
+    // no tokens: the single chunk is empty, but its row of the table is still read
+    hipLaunchKernelGGL(align_count_kernel, dim3(1), dim3(kThreads), 0, s, ids, (int64_t)0, E, chunk_counts);
+  }
+  hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s, ids,
+                     numel, E, block, chunk_counts, (int)chunks, kRouteChunkTokens * K, sorted_ids,
+                     sorted_cap, expert_ids, expert_ids_cap, counts, num_post_pad);
   return launch_status();
 }

@@ -35,14 +35,15 @@ __device__ __forceinline__ void row_step_max(uint32_t& key, uint32_t& tag) {
   tag = take ? ot : tag;
 }
 
+// Routes one token on the calling DPP row: lane r < K of the row stores the r-th selected
+// probability and expert and gets that expert back (other lanes and dead rows: -1).
 template <int VPL>
-__global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
-    const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
-    int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok) {
+__device__ __forceinline__ int32_t route_token(const float* __restrict__ logits,
+                                               float* __restrict__ weights,
+                                               int32_t* __restrict__ ids, int64_t token, bool live,
+                                               int E, int K, int64_t ld, int renorm, int vec_ok) {
   const int lane16 = threadIdx.x & 15;
-  const int64_t token = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   // every lane of a row takes the same branch; DPP rows never straddle tokens
-  const bool live = token < T;
   const float NEG_INF = -__builtin_inff();
 
   float v[VPL];
@@ -126,10 +127,64 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
     const float w = renorm ? my_w / wsum : my_w;
     weights[token * K + lane16] = w;
     ids[token * K + lane16] = my_id;
+    return my_id;
   }
+  return -1;
+}
+
+template <int VPL>
+__global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
+    const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
+    int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok) {
+  const int64_t token = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  route_token<VPL>(logits, weights, ids, token, token < T, E, K, ld, renorm, vec_ok);
+}
+
+// The router fused with the first step of the expert alignment: a workgroup of 1024 threads
+// routes kRouteChunkTokens consecutive tokens (64 per pass) and histograms the experts it
+// selected in LDS, then writes one row of the alignment's [chunks, E] count table -- the row of
+// the chunk made of exactly those tokens' K * kRouteChunkTokens flat routing slots.  Integer
+// LDS adds only, so the row does not depend on the order of execution.
+template <int VPL>
+__global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
+    const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
+    int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok,
+    int32_t* __restrict__ chunk_counts) {
+  __shared__ int32_t hist[256];
+  for (int e = threadIdx.x; e < E; e += 1024) hist[e] = 0;
+  __syncthreads();
+  const int64_t first = (int64_t)blockIdx.x * kRouteChunkTokens;
+#pragma unroll
+  for (int pass = 0; pass < kRouteChunkTokens / 64; ++pass) {
+    const int64_t token = first + pass * 64 + (threadIdx.x >> 4);
+    const int32_t e = route_token<VPL>(logits, weights, ids, token, token < T, E, K, ld, renorm, vec_ok);
+    if (e >= 0) atomicAdd(&hist[e], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 1024) chunk_counts[(int64_t)blockIdx.x * E + e] = hist[e];
 }
 
 }  // namespace
+
+// launch of the fused router + chunk histogram (used by the fused entry point of the alignment)
+int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
+                              int K, int64_t ld_logits, int renormalize, int32_t* chunk_counts,
+                              hipStream_t s) {
+  const dim3 grid((uint32_t)ceil_div(T, kRouteChunkTokens)), block(1024);
+  const bool a16 = aligned16(logits) && (ld_logits % 4 == 0);
+  if (E <= 64) {
+    hipLaunchKernelGGL(moe_topk_softmax_count_kernel<4>, grid, block, 0, s, logits, weights, ids, T,
+                       E, K, ld_logits, renormalize, (int)(a16 && E == 64), chunk_counts);
+  } else if (E <= 128) {
+    hipLaunchKernelGGL(moe_topk_softmax_count_kernel<8>, grid, block, 0, s, logits, weights, ids, T,
+                       E, K, ld_logits, renormalize, (int)(a16 && E == 128), chunk_counts);
+  } else {
+    hipLaunchKernelGGL(moe_topk_softmax_count_kernel<16>, grid, block, 0, s, logits, weights, ids, T,
+                       E, K, ld_logits, renormalize, (int)(a16 && E == 256), chunk_counts);
+  }
+  return launch_status();
+}
+
 }  // namespace dlb
 
 extern "C" int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids,

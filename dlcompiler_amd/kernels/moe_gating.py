@@ -85,3 +85,56 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     if return_counts:
         return sorted_ids, expert_ids, num_post, counts
     return sorted_ids, expert_ids, num_post
+
+
+_FUSED_MAX_TOKENS = 32768  # beyond this the fused entry point declines (DLB_ERR_UNSUPPORTED)
+
+
+def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_experts: int = None,
+                           renormalize: bool = True):
+    """:func:`moe_topk_softmax` followed by :func:`moe_align_block_size` on its ids, as one
+    native call of two launches (the router also produces the alignment's per-chunk expert
+    counts).  Returns ``(weights, ids, sorted_token_ids, expert_ids, num_tokens_post_padded)``,
+    bit for bit what the two functions return.  More than 32768 tokens, or ``num_experts``
+    different from the router's expert count, take the two separate calls.
+    """
+    assert logits.dim() == 2
+    _lib.require_cuda(logits)
+    T, E = logits.shape
+    if num_experts is None:
+        num_experts = E
+    if not 1 <= k <= E:
+        raise ValueError(f"need 1 <= k <= num_experts, got k={k}, E={E}")
+    if block_size < 1:
+        raise ValueError("block_size must be positive")
+    if T > _FUSED_MAX_TOKENS or num_experts != E or k > 16 or E > 256:
+        weights, ids = moe_topk_softmax(logits, k, renormalize)
+        return (weights, ids) + tuple(moe_align_block_size(ids, block_size, num_experts))
+    if logits.dtype != torch.float32:
+        logits = logits.float()
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    dev = logits.device
+    numel = T * k
+    cap = numel + E * (block_size - 1)
+    nblk = max(1, -(-cap // block_size))
+    lib = _lib.load()
+    ws_words = max((lib.dlb_moe_topk_softmax_align_ws_bytes(T, E) + 3) // 4, 1)
+    # one allocation of 4-byte words, carved into the results and the scratch
+    sizes = (numel, numel, cap, nblk, 1, ws_words)
+    offs, total = [], 0
+    for n in sizes:
+        offs.append(total)
+        total += (n + 3) & ~3
+    buf = torch.empty((total,), dtype=torch.int32, device=dev)
+    w_raw, ids, sorted_ids, expert_ids, num_post, ws = (buf[o:o + n] for o, n in zip(offs, sizes))
+    weights = w_raw.view(torch.float32).view(T, k)
+    ids = ids.view(T, k)
+    with _lib.device_guard(dev):
+        st = lib.dlb_moe_topk_softmax_align_f32(
+            logits.data_ptr(), weights.data_ptr(), ids.data_ptr(), T, E, k,
+            logits.stride(0) if T > 1 else E, int(bool(renormalize)), block_size,
+            sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk, None, num_post.data_ptr(),
+            ws.data_ptr(), ws.numel() * 4, _lib.current_stream_ptr(dev))
+    _lib.check(st, "dlb_moe_topk_softmax_align_f32")
+    return weights, ids, sorted_ids, expert_ids, num_post

@@ -91,6 +91,23 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
                              void* ws, size_t ws_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Router and alignment in one call (two launches instead of three): the outputs of
+ * dlb_moe_topk_softmax_f32 followed by dlb_moe_align_block_size on its ids, bit for bit.
+ * The same reference lines as the two calls above: the router of
+ * tests/kernels/test_fused_moe.py:213-216 + kernels/fused_moe.py:322-323 and the routing
+ * bookkeeping of kernels/fused_moe.py:238-293,314-320.
+ * Arguments as in those two functions (numel = T * K); ws of
+ * dlb_moe_topk_softmax_align_ws_bytes(T, E) bytes.  Returns DLB_ERR_UNSUPPORTED for more than
+ * 32768 tokens: make the two calls then.
+ * ---------------------------------------------------------------------------------------- */
+size_t dlb_moe_topk_softmax_align_ws_bytes(int64_t T, int E);
+int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t* ids, int64_t T,
+                                   int E, int K, int64_t ld_logits, int renormalize, int block,
+                                   int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids,
+                                   int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
+                                   void* ws, size_t ws_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Paged decode attention: one query token per sequence against a paged KV cache, GQA.
  * Replaces the decode branch of paged_attention_fwd, kernels/paged_attention.py:604-671
  * (_fwd_grouped_split_kernel :45-234 and _reduce_split_kernel :238-285).

@@ -121,3 +121,30 @@ def test_end_to_end_config2(dev):
     assert torch.equal(e.cpu(), re_) and tot.item() == rtot.item()
     torch.testing.assert_close(w.cpu(), rw, rtol=1e-6, atol=0)
     np.testing.assert_allclose(w.cpu().sum(-1).numpy(), 1.0, atol=3e-7)
+
+
+@pytest.mark.parametrize("T,E,k,block", [(16384, 64, 6, 64), (1, 64, 6, 64), (127, 8, 2, 16),
+                                         (128, 60, 6, 64), (129, 64, 8, 128), (333, 160, 6, 32),
+                                         (5000, 256, 16, 64), (32768, 16, 4, 64), (0, 64, 6, 64),
+                                         (40000, 64, 6, 64)])   # the last one: the two-call path
+@pytest.mark.parametrize("renorm", [True, False])
+def test_fused_router_and_alignment_equals_the_two_calls(dev, T, E, k, block, renorm):
+    from dlcompiler_amd.kernels.moe_gating import (moe_align_block_size, moe_topk_softmax,
+                                                   moe_topk_softmax_align)
+
+    g = torch.Generator().manual_seed(T + E)
+    logits = torch.randn((T, E), generator=g).to(dev)
+    if T > 3:
+        logits[2] = 0.0                                       # a row of ties
+    w, ids, sorted_ids, expert_ids, npad = moe_topk_softmax_align(logits, k, block, renormalize=renorm)
+    rw, rids = moe_topk_softmax(logits, k, renormalize=renorm)
+    rs, re_, rn = moe_align_block_size(rids, block, E)
+    assert w.dtype == torch.float32 and ids.dtype == torch.int32 and w.shape == (T, k)
+    assert torch.equal(ids, rids) and torch.equal(w, rw)
+    assert torch.equal(npad, rn) and torch.equal(sorted_ids, rs) and torch.equal(expert_ids, re_)
+    if T > 0:   # and against the oracle, not only against the other native path
+        ow, oids = og.topk_softmax(logits.cpu(), k, renormalize=renorm)
+        assert torch.equal(ids.cpu(), oids)
+        os_, oe, otot, _ = og.align_block_size(oids, block, E)
+        assert torch.equal(sorted_ids.cpu(), os_) and torch.equal(expert_ids.cpu(), oe)
+        assert int(npad.item()) == int(otot.item())
