@@ -152,13 +152,6 @@ struct MoeGemmParams {
 #define DLB_MOE_OCC 2
 #endif
 
-#ifdef DLB_TIMING
-__device__ unsigned long long dbg_t[4096];
-__device__ int dbg_n;
-#define DLB_T() do { if ((blockIdx.x == 1032 || blockIdx.x == 2064) && threadIdx.x == 0 && dbg_n < 2040) { dbg_t[2 * dbg_n] = clock64(); dbg_t[2 * dbg_n + 1] = wall_clock64(); ++dbg_n; } } while (0)
-#else
-#define DLB_T() do { } while (0)
-#endif
 
 __device__ __forceinline__ i32x8 cat8(const u32x4& lo, const u32x4& hi) {
   return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3],
@@ -246,7 +239,6 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   const int e = e_global - p.expert_offset;
   if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
 
-  DLB_T();
   int out_sid[2] = {0, 0};
   float out_rw[2] = {0.0f, 0.0f};
   if (!GATED) {
@@ -311,9 +303,6 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   const unsigned int sc_dst0 = lds_addr(sc_lds) + wave * kScWave;
   // all direct-to-LDS operations of chunk kc (clamped past the end: the count per chunk is fixed)
   auto issue_x = [&](int kc, int slot) {
-#ifdef DLB_ABL_NOX
-    if (kc > 2) return;
-#endif
     const int kcc = min(kc, KC - 1);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -324,15 +313,6 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   };
   // weight unit (kc, ct); past the end every lane re-reads the expert's first 16 bytes
   auto issue_w = [&](int kc, int ct, u32x4 (&b)[4]) {
-#ifdef DLB_ABL_NOW
-    if (kc > 1) {
-      asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-      return;
-    }
-#endif
-#ifdef DLB_ABL_L2
-    kc &= 1;
-#endif
     const bool live = kc < KC;
     const unsigned char* sbase = uniform_ptr(wbase + (live ? kc : 0) * kWChunk);
     load_w_unit<WL>(b, live ? woff[ct] : 0u, sbase);
@@ -348,16 +328,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   // two waves' strips apart
   const unsigned char* as_mine = sc_lds + (j >> 4) * kScWave + (j & 15) * 4;
   const unsigned char* ws_mine = sc_lds + wave * kScWave + 64;
-#ifdef DLB_ABL_NOREAD
-  bool abl_started = false;
-#endif
   auto read_x = [&](int slot, int rt, u32x4 (&x)[4], float& as) {
-#ifdef DLB_ABL_NOREAD
-    if (abl_started) {
-      asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(as));
-      return;
-    }
-#endif
 #pragma unroll
     for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(x_lds + slot * kXSlot + rt * 4096 + xf[q]);
     as = QT == 0 ? *(const float*)(as_mine + slot * kScSlot + rt * (2 * kScWave)) : 1.0f;
@@ -429,7 +400,6 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
   issue_w(1, 1, wr[1][1]);
   wait_vm<16 + 2 * D>();  // X(0) landed
   __syncthreads();
-  DLB_T();
   read_x(0, 0, x0, as0);
 
   int x_cur = 0, x_nxt = 1, x_tgt = 2;  // slots of chunks k, k + 1, k + 2
@@ -451,12 +421,7 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     __builtin_amdgcn_sched_barrier(0);
     issue_w(k + 2, 0, wr[P][0]);
     wait_vm<16 + D>();  // this wave's part of X(k + 1) landed
-#ifdef DLB_ABL_NOREAD
-    abl_started = true;
-#endif
-#ifndef DLB_ABL_NOBAR
     __syncthreads();    // X(k + 1) complete; every wave is done reading X(k)
-#endif
     issue_x(k + 3, x_cur);
     wait_w_unit<12 + 2 * D>(wr[P][1]);  // W(k, ct 1) landed
     __builtin_amdgcn_sched_barrier(0);
@@ -491,7 +456,6 @@ __device__ __forceinline__ void moe_gemm_fp8_tile(const MoeGemmParams& p, const 
     for (int r = 0; r < 16; ++r) acc[1][1][r] += pp[r] * psc;
   }
 
-  DLB_T();
 
   // ---- epilogues: lane holds token (32*rt + j), columns ncol[ct] + 8*(r/4) + 4*h + r%4.
   // A swap between the lane halves turns two 4-column runs into one 8-column run per lane.
@@ -641,7 +605,6 @@ __global__ __launch_bounds__(256, DLB_MOE_OCC) void moe_gemm_fp8_kernel(const Mo
     const int logical = xcd * per_xcd + i;
     if (logical < p.grid_real) moe_gemm_fp8_tile<GATED, DT, QT, WL>(p, logical);
     __syncthreads();  // the tile's LDS is reused by the next one
-    DLB_T();
   }
 }
 
@@ -697,7 +660,6 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   const int e = e_global - p.expert_offset;
   if (e_global < 0 || e < 0 || e >= p.num_local) return;  // tail block / expert of another shard
 
-  DLB_T();
   if (tid < BM) sid_lds[tid] = sid_mine;
 
   // source row of tile row r whose routing slot is sid (gated: the slot's token; pad slots read
@@ -779,27 +741,12 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     xf[q] = rg * (64 * 128) + (f0 ^ (q << 5));
   }
   const float* as_base = &as_lds[0][64 * rg + j];
-#ifdef DLB_ABL_NOREAD
-  bool first_reads = true;
-#endif
   auto read_w = [&](int slot, int ct, u32x4 (&b)[4]) {
-#ifdef DLB_ABL_NOREAD
-    if (!first_reads) {
-      asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-      return;
-    }
-#endif
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       b[q] = *(const u32x4*)(w_lds + slot * kWSlot + ct * kCtStride + wf[q]);
   };
   auto read_x = [&](int slot, int kc, int rt, u32x4 (&x)[4], float& as) {
-#ifdef DLB_ABL_NOREAD
-    if (!first_reads) {
-      asm volatile("" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(as));
-      return;
-    }
-#endif
 #pragma unroll
     for (int q = 0; q < 4; ++q) x[q] = *(const u32x4*)(x_lds + slot * kXSlot + rt * 4096 + xf[q]);
     as = QT == 0 ? as_base[(kc & (kSC - 1)) * BM + 32 * rt] : 1.0f;
@@ -843,7 +790,6 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     else __builtin_amdgcn_s_waitcnt(0x0F70);              // vmcnt(0)
   }
   __syncthreads();
-  DLB_T();
   read_w(0, 0, ba);
   read_x(0, 0, 0, x0, as0);
   if (QT == 0) {
@@ -899,9 +845,6 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
   // step of MFMAs to hide behind.
   for (int kc = 0; kc < KC; ++kc) {
     const bool more = kc + 1 < KC;
-#ifdef DLB_ABL_NOREAD
-    first_reads = kc == 0;
-#endif
     read_w(w_cur, 1, bb);
     read_x(x_cur, kc, 1, x1, as1);
     __builtin_amdgcn_sched_barrier(0);
@@ -913,18 +856,14 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
       // chunk kc + 1 has landed once every wave's own loads of it are back
       if (kc + 2 < KC) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);  // W(kc + 2) may still fly
       else __builtin_amdgcn_s_waitcnt(0x0F70);
-#ifndef DLB_ABL_NOBAR
       __syncthreads();
-#endif
       if (QT == 0 && ((kc + 1) & (kSC - 1)) == 0) {
         // rare (K > 2048 bytes): next tile of activation scales; every wave has fetched its
         // scales of chunk kc before the barrier above
         load_scales(kc + 1);
         __syncthreads();
       }
-#ifndef DLB_ABL_NODMA
       if (kc + 2 < KC) issue_x(kc + 2, x_tgt);
-#endif
       read_w(w_nxt, 0, ba);
       if (QT == 0) {
         wsn[0] = ws_row0[(kc + 1) & (kSC - 1)];
@@ -936,9 +875,7 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
     __builtin_amdgcn_sched_barrier(0);
     // the weights of chunk kc + 3 (least urgent) go out a step after the activations, which
     // spreads the workgroup's requests; still issued after X(kc + 2), as the waits assume
-#ifndef DLB_ABL_NODMA
     if (kc + 3 < KC) issue_w(kc + 3, w_cur);
-#endif
     if (more) read_x(x_nxt, kc + 1, 0, x0, as0);
     __builtin_amdgcn_sched_barrier(0);
     step(bb, x1, acc[1][1], acc[0][1], as1 * wsc[1]);
@@ -960,7 +897,6 @@ __device__ __forceinline__ void moe_gemm_wide_tile(const MoeGemmParams& p, const
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[1][1][r] += pp[r] * psc;
   }
-  DLB_T();
 
   // ---- epilogues: lane holds slot row (64 rg + 32 rt + j), columns (tile ct) + 8 (r / 4) +
   // 4 h + r % 4; a swap between the lane halves gives each lane 8 adjacent columns.
@@ -1096,7 +1032,6 @@ __global__ __launch_bounds__(512, 1) void moe_gemm_wide_kernel(const MoeGemmPara
     const int logical = xcd * per_xcd + i;
     if (logical < p.grid_real) moe_gemm_wide_tile<GATED, DT, QT>(p, logical);
     __syncthreads();  // the tile's LDS is reused by the next one
-    DLB_T();
   }
 }
 
@@ -1130,15 +1065,6 @@ __global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restri
 }  // namespace
 }  // namespace dlb
 
-#ifdef DLB_TIMING
-extern "C" int dlb_debug_read(unsigned long long* dst, int* n) {
-  int z = 0;
-  if (hipMemcpyFromSymbol(dst, HIP_SYMBOL(dlb::dbg_t), sizeof(unsigned long long) * 4096) != hipSuccess) return -1;
-  if (hipMemcpyFromSymbol(n, HIP_SYMBOL(dlb::dbg_n), sizeof(int)) != hipSuccess) return -1;
-  if (hipMemcpyToSymbol(HIP_SYMBOL(dlb::dbg_n), &z, sizeof(int)) != hipSuccess) return -1;
-  return 0;
-}
-#endif
 
 extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
                                              int K, int64_t ld_x, int64_t ld_q, int64_t ld_s,
