@@ -35,18 +35,15 @@ __device__ __forceinline__ void row_step_max(uint32_t& key, uint32_t& tag) {
   tag = take ? ot : tag;
 }
 
-// Routes one token on the calling DPP row: lane r < K of the row stores the r-th selected
-// probability and expert and gets that expert back (other lanes and dead rows: -1).
+// The logits of one token, VPL consecutive experts per lane of its DPP row (-inf past E and for
+// dead rows).
 template <int VPL>
-__device__ __forceinline__ int32_t route_token(const float* __restrict__ logits,
-                                               float* __restrict__ weights,
-                                               int32_t* __restrict__ ids, int64_t token, bool live,
-                                               int E, int K, int64_t ld, int renorm, int vec_ok) {
+__device__ __forceinline__ void load_token_logits(const float* __restrict__ logits, int64_t token,
+                                                  bool live, int E, int64_t ld, int vec_ok,
+                                                  float (&v)[VPL]) {
   const int lane16 = threadIdx.x & 15;
   // every lane of a row takes the same branch; DPP rows never straddle tokens
   const float NEG_INF = -__builtin_inff();
-
-  float v[VPL];
   const int e0 = lane16 * VPL;
   if (live && vec_ok) {
     const f32x4* p = reinterpret_cast<const f32x4*>(logits + token * ld + e0);
@@ -63,6 +60,16 @@ __device__ __forceinline__ int32_t route_token(const float* __restrict__ logits,
     for (int j = 0; j < VPL; ++j)
       v[j] = (live && e0 + j < E) ? logits[token * ld + e0 + j] : NEG_INF;
   }
+}
+
+// Routes one token, whose logits the calling DPP row holds: lane r < K of the row stores the
+// r-th selected probability and expert and gets that expert back (other lanes and dead rows: -1).
+template <int VPL>
+__device__ __forceinline__ int32_t route_token(const float (&v)[VPL], float* __restrict__ weights,
+                                               int32_t* __restrict__ ids, int64_t token, bool live,
+                                               int E, int K, int renorm) {
+  const int lane16 = threadIdx.x & 15;
+  const int e0 = lane16 * VPL;
 
   // softmax statistics: p_e = exp(l_e - max) / sum
   float mx = v[0];
@@ -137,7 +144,9 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
     const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
     int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok) {
   const int64_t token = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  route_token<VPL>(logits, weights, ids, token, token < T, E, K, ld, renorm, vec_ok);
+  float v[VPL];
+  load_token_logits<VPL>(logits, token, token < T, E, ld, vec_ok, v);
+  route_token<VPL>(v, weights, ids, token, token < T, E, K, renorm);
 }
 
 // The router fused with the first step of the expert alignment: a workgroup of 1024 threads
@@ -154,10 +163,17 @@ __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
   for (int e = threadIdx.x; e < E; e += 1024) hist[e] = 0;
   __syncthreads();
   const int64_t first = (int64_t)blockIdx.x * kRouteChunkTokens;
+  constexpr int kPasses = kRouteChunkTokens / 64;
+  float v[kPasses][VPL];
 #pragma unroll
-  for (int pass = 0; pass < kRouteChunkTokens / 64; ++pass) {
+  for (int pass = 0; pass < kPasses; ++pass) {  // all loads first: one memory round trip
     const int64_t token = first + pass * 64 + (threadIdx.x >> 4);
-    const int32_t e = route_token<VPL>(logits, weights, ids, token, token < T, E, K, ld, renorm, vec_ok);
+    load_token_logits<VPL>(logits, token, token < T, E, ld, vec_ok, v[pass]);
+  }
+#pragma unroll
+  for (int pass = 0; pass < kPasses; ++pass) {
+    const int64_t token = first + pass * 64 + (threadIdx.x >> 4);
+    const int32_t e = route_token<VPL>(v[pass], weights, ids, token, token < T, E, K, renorm);
     if (e >= 0) atomicAdd(&hist[e], 1);
   }
   __syncthreads();
