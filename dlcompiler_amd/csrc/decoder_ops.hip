@@ -125,14 +125,14 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(
   for (int q = 0; q < kMaxVec; ++q) {
     const int i = q * kNormThreads + threadIdx.x;
     if (i < nvec) {
-      v[q] = *(const u32x4*)(x + row * ld_x + 8 * i);
+      v[q] = __builtin_nontemporal_load((const u32x4*)(x + row * ld_x + 8 * i));  // streamed once
       if (ADD) {
-        const u32x4 r = *(const u32x4*)(res + row * ld_res + 8 * i);
+        const u32x4 r = __builtin_nontemporal_load((const u32x4*)(res + row * ld_res + 8 * i));
 #pragma unroll
         for (int k = 0; k < 4; ++k)
           v[q][k] = Elem<DT>::pack(Elem<DT>::lo(v[q][k]) + Elem<DT>::lo(r[k]),
                                    Elem<DT>::hi(v[q][k]) + Elem<DT>::hi(r[k]));
-        *(u32x4*)(out_res + row * ld_out_res + 8 * i) = v[q];
+        __builtin_nontemporal_store(v[q], (u32x4*)(out_res + row * ld_out_res + 8 * i));
       }
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(
         o[k] = Elem<DT>::pack(Elem<DT>::lo(nrm) * Elem<DT>::lo(wv[k]),
                               Elem<DT>::hi(nrm) * Elem<DT>::hi(wv[k]));
       }
-      *(u32x4*)(out + row * ld_out + 8 * i) = o;
+      __builtin_nontemporal_store(o, (u32x4*)(out + row * ld_out + 8 * i));
     }
   }
 }
