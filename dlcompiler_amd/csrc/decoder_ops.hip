@@ -189,7 +189,9 @@ __global__ __launch_bounds__(256) void rotary_kernel(
       src = k + t * k_st + (int64_t)(h - Hq) * k_sh;
       dst = ko + t * ko_st + (int64_t)(h - Hq) * ko_sh;
     }
-    const u32x4 xl = *(const u32x4*)(src + 8 * c), xh = *(const u32x4*)(src + half + 8 * c);
+    // q/k are streamed once (non-temporal); cos/sin are shared by every head of the token
+    const u32x4 xl = __builtin_nontemporal_load((const u32x4*)(src + 8 * c));
+    const u32x4 xh = __builtin_nontemporal_load((const u32x4*)(src + half + 8 * c));
     const u32x4 cl = *(const u32x4*)(cos_ + t * cs_st + 8 * c);
     const u32x4 ch = *(const u32x4*)(cos_ + t * cs_st + half + 8 * c);
     const u32x4 sl = *(const u32x4*)(sin_ + t * cs_st + 8 * c);
@@ -204,8 +206,8 @@ __global__ __launch_bounds__(256) void rotary_kernel(
       oh[j] = Elem<DT>::pack(h0 * Elem<DT>::lo(ch[j]) + l0 * Elem<DT>::lo(sh[j]),
                              h1 * Elem<DT>::hi(ch[j]) + l1 * Elem<DT>::hi(sh[j]));
     }
-    *(u32x4*)(dst + 8 * c) = ol;
-    *(u32x4*)(dst + half + 8 * c) = oh;
+    __builtin_nontemporal_store(ol, (u32x4*)(dst + 8 * c));
+    __builtin_nontemporal_store(oh, (u32x4*)(dst + half + 8 * c));
   }
 }
 
