@@ -101,7 +101,30 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
 
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * SM::stage];
 
-  const int seq = blockIdx.z;
+  // Paged (chunked) prefill: a sequence's cost is set by its history, which differs widely
+  // between the sequences of a batch while the grid holds only a few workgroups per slot, so
+  // the sequences are walked longest context first (blockIdx.z = rank, not index): the long
+  // ones start in the first round and the short ones fill in behind them.
+  int seq = blockIdx.z;
+  if (PAGED && gridDim.z > 1 && gridDim.z <= kThreads) {
+    __shared__ int32_t rank_key[kThreads];
+    __shared__ int32_t rank_seq;
+    const int nb = gridDim.z;
+    const int t = threadIdx.x;
+    const int key = t < nb ? p.kv_len[t] : 0;
+    rank_key[t] = key;
+    __syncthreads();
+    if (t < nb) {
+      int rank = 0;
+      for (int j = 0; j < nb; ++j) {
+        const int kj = rank_key[j];
+        rank += (kj > key || (kj == key && j < t)) ? 1 : 0;
+      }
+      if (rank == (int)blockIdx.z) rank_seq = t;  // ranks are a permutation: exactly one writer
+    }
+    __syncthreads();
+    seq = __builtin_amdgcn_readfirstlane(rank_seq);
+  }
   const int L = p.seq_len[seq];
   const int qtile = gridDim.y - 1 - blockIdx.y;  // heaviest tiles first
   const int q0 = qtile * kBlockM;
