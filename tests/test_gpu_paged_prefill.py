@@ -123,3 +123,15 @@ def test_grid_larger_than_needed_and_rejects(dev):
         paged_attention_fwd(q, kc, kc, torch.empty_like(q), torch.zeros(2, 2, dtype=torch.int32, device=dev),
                             torch.tensor([0, 4], device=dev), torch.tensor([4, 4], device=dev),
                             torch.tensor([4, 4], device=dev), 4)
+
+
+# the kernel walks the sequences longest context first when the batch fits one workgroup's
+# ranking pass (<= 256 sequences) and in index order beyond: both sides of that limit, with
+# equal contexts (rank ties) among them
+@pytest.mark.parametrize("nseq", [2, 255, 256, 257, 600])
+def test_many_sequences_any_order(dev, nseq):
+    g = torch.Generator().manual_seed(nseq)
+    q_lens = torch.randint(0, 6, (nseq,), generator=g).tolist()
+    hist = torch.randint(0, 40, (nseq,), generator=g).tolist()
+    hist[1] = hist[0] + q_lens[0] - q_lens[1] if hist[0] + q_lens[0] >= q_lens[1] else hist[1]
+    _run_case(dev, q_lens, hist, 4, 2, 128, 16, torch.bfloat16, seed=nseq)
