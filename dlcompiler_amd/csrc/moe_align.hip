@@ -199,6 +199,21 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   const int wave = tid / kWave;
   const int me = blockIdx.x;
 
+  // this chunk's first ids are requested before the count table is reduced (they do not depend
+  // on it), each later tile's while the tile before it is placed
+  const int64_t begin = (int64_t)me * chunk_ids;  // chunk_ids flat ids per chunk (kChunk by default)
+  const int64_t end = begin + chunk_ids < numel ? begin + chunk_ids : numel;
+  auto load_expert = [&](int64_t tile) -> int32_t {
+    const int64_t i = tile + tid;
+    int32_t e = -1;
+    if (i < end) {
+      e = ids[i];
+      if (e < 0 || e >= E) e = -1;
+    }
+    return e;
+  };
+  int32_t e_next = load_expert(begin);
+
   // totals and the part of them that lies in earlier chunks: sub-group q = tid / E' (E' = E
   // rounded up to a whole wave) sums a slice of the chunk rows for expert tid % E', the slices
   // meet in LDS (wave_cnt doubles as the scratch for that before it is cleared)
@@ -210,6 +225,7 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
     const int c0 = q * per, c1 = min(c0 + per, chunks);
     int32_t total = 0, before_part = 0;
     if (e < E && q < groups) {
+#pragma unroll 8  // independent loads: eight rows in flight instead of one round trip each
       for (int c = c0; c < c1; ++c) {
         const int32_t n = chunk_counts[(int64_t)c * E + e];
         total += n;
@@ -271,16 +287,11 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   }
   __syncthreads();
 
-  const int64_t begin = (int64_t)me * chunk_ids;  // chunk_ids flat ids per chunk (kChunk by default)
-  const int64_t end = begin + chunk_ids < numel ? begin + chunk_ids : numel;
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   for (int64_t tile = begin; tile < end; tile += kThreads) {  // uniform trip count
     const int64_t i = tile + tid;
-    int32_t e = -1;
-    if (i < end) {
-      e = ids[i];
-      if (e < 0 || e >= E) e = -1;
-    }
+    const int32_t e = e_next;
+    e_next = load_expert(tile + kThreads);
     // lanes of this wave holding the same expert: intersect ballots over the 9 key bits
     const uint32_t key = (uint32_t)e & 0x1ffu;
     uint64_t peers = ~0ull;
