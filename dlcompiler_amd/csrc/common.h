@@ -190,11 +190,14 @@ __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // tokens per workgroup of the fused router + chunk-histogram kernel = tokens per alignment chunk
-// when the two run as one pipeline
-constexpr int kRouteChunkTokens = 128;  // 64 and 256 measured no faster at 16384 tokens
+// when the two run as one pipeline: 64 (one pass; twice the workgroups, 8 instead of 12 us for
+// the router at 16384 tokens) while that keeps the count table within the 256 rows the fused
+// placement kernel reduces, else 128 (two passes)
+constexpr int kRouteMaxChunks = 256;
+inline int route_chunk_tokens(int64_t T) { return (T + 63) / 64 <= kRouteMaxChunks ? 64 : 128; }
 int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
-                              int K, int64_t ld_logits, int renormalize, int32_t* chunk_counts,
-                              hipStream_t s);
+                              int K, int64_t ld_logits, int renormalize, int chunk_tokens,
+                              int32_t* chunk_counts, hipStream_t s);
 
 // status of the launch just issued on this thread
 inline int launch_status() { return hipGetLastError() == hipSuccess ? DLB_OK : DLB_ERR_LAUNCH; }

@@ -184,6 +184,7 @@ __global__ __launch_bounds__(kThreads) void align_place_kernel(
 // one extra workgroup emits what the scan kernel emits (counts, block -> expert ids, pad slots,
 // tails, padded total).  The table is only read here.
 constexpr int kFusedChunks = 256;
+static_assert(kFusedChunks == kRouteMaxChunks, "the fused router sizes its chunks for this table");
 
 __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
     const int32_t* __restrict__ ids, int64_t numel, int E, int block,
@@ -369,12 +370,12 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
 
 // ---------------------------------------------------------------------------------------
 // Router and alignment as one pipeline of two launches: the router kernel also writes the
-// per-chunk expert counts (a chunk = the K routing slots of kRouteChunkTokens consecutive
+// per-chunk expert counts (a chunk = the K routing slots of route_chunk_tokens(T) consecutive
 // tokens), so the alignment's own counting pass over the ids is not needed.
 // ---------------------------------------------------------------------------------------
 extern "C" size_t dlb_moe_topk_softmax_align_ws_bytes(int64_t T, int E) {
   if (T < 0 || E < 1) return 0;
-  const int64_t chunks = T > 0 ? dlb::ceil_div(T, dlb::kRouteChunkTokens) : 1;
+  const int64_t chunks = T > 0 ? dlb::ceil_div(T, dlb::route_chunk_tokens(T)) : 1;
   return (size_t)chunks * (size_t)E * sizeof(int32_t);
 }
 
@@ -390,7 +391,8 @@ extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weight
   if (K > 16 || E > kMaxE) return DLB_ERR_UNSUPPORTED;
   const int64_t numel = T * K;
   if (numel + (int64_t)E * block >= (int64_t)0x7fffffff) return DLB_ERR_UNSUPPORTED;
-  const int64_t chunks = T > 0 ? ceil_div(T, kRouteChunkTokens) : 1;
+  const int chunk_tokens = route_chunk_tokens(T);
+  const int64_t chunks = T > 0 ? ceil_div(T, chunk_tokens) : 1;
   // larger inputs take the two separate entry points (their scan runs as its own launch)
   if (chunks > kFusedChunks) return DLB_ERR_UNSUPPORTED;
   if (!sorted_ids || !expert_ids || !num_post_pad || (T > 0 && (!logits || !weights || !ids)))
@@ -402,14 +404,14 @@ extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weight
   int32_t* chunk_counts = (int32_t*)ws;
   if (T > 0) {
     const int st = launch_topk_softmax_count(logits, weights, ids, T, E, K, ld_logits, renormalize,
-                                             chunk_counts, s);
+                                             chunk_tokens, chunk_counts, s);
     if (st != DLB_OK) return st;
   } else {
     // no tokens: the single chunk is empty, but its row of the table is still read
     hipLaunchKernelGGL(align_count_kernel, dim3(1), dim3(kThreads), 0, s, ids, (int64_t)0, E, chunk_counts);
   }
   hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s, ids,
-                     numel, E, block, chunk_counts, (int)chunks, kRouteChunkTokens * K, sorted_ids,
+                     numel, E, block, chunk_counts, (int)chunks, chunk_tokens * K, sorted_ids,
                      sorted_cap, expert_ids, expert_ids_cap, counts, num_post_pad);
   return launch_status();
 }

@@ -150,11 +150,11 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
 }
 
 // The router fused with the first step of the expert alignment: a workgroup of 1024 threads
-// routes kRouteChunkTokens consecutive tokens (64 per pass) and histograms the experts it
-// selected in LDS, then writes one row of the alignment's [chunks, E] count table -- the row of
-// the chunk made of exactly those tokens' K * kRouteChunkTokens flat routing slots.  Integer
-// LDS adds only, so the row does not depend on the order of execution.
-template <int VPL>
+// routes 64 * PASSES consecutive tokens (64 per pass) and histograms the experts it selected
+// in LDS, then writes one row of the alignment's [chunks, E] count table -- the row of the
+// chunk made of exactly those tokens' K * 64 * PASSES flat routing slots.  Integer LDS adds
+// only, so the row does not depend on the order of execution.
+template <int VPL, int PASSES>
 __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
     const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
     int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok,
@@ -162,16 +162,15 @@ __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
   __shared__ int32_t hist[256];
   for (int e = threadIdx.x; e < E; e += 1024) hist[e] = 0;
   __syncthreads();
-  const int64_t first = (int64_t)blockIdx.x * kRouteChunkTokens;
-  constexpr int kPasses = kRouteChunkTokens / 64;
-  float v[kPasses][VPL];
+  const int64_t first = (int64_t)blockIdx.x * (64 * PASSES);
+  float v[PASSES][VPL];
 #pragma unroll
-  for (int pass = 0; pass < kPasses; ++pass) {  // all loads first: one memory round trip
+  for (int pass = 0; pass < PASSES; ++pass) {  // all loads first: one memory round trip
     const int64_t token = first + pass * 64 + (threadIdx.x >> 4);
     load_token_logits<VPL>(logits, token, token < T, E, ld, vec_ok, v[pass]);
   }
 #pragma unroll
-  for (int pass = 0; pass < kPasses; ++pass) {
+  for (int pass = 0; pass < PASSES; ++pass) {
     const int64_t token = first + pass * 64 + (threadIdx.x >> 4);
     const int32_t e = route_token<VPL>(v[pass], weights, ids, token, token < T, E, K, renorm);
     if (e >= 0) atomicAdd(&hist[e], 1);
@@ -182,22 +181,29 @@ __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
 
 }  // namespace
 
-// launch of the fused router + chunk histogram (used by the fused entry point of the alignment)
+// launch of the fused router + chunk histogram (used by the fused entry point of the alignment);
+// chunk_tokens is 64 or 128
 int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
-                              int K, int64_t ld_logits, int renormalize, int32_t* chunk_counts,
-                              hipStream_t s) {
-  const dim3 grid((uint32_t)ceil_div(T, kRouteChunkTokens)), block(1024);
+                              int K, int64_t ld_logits, int renormalize, int chunk_tokens,
+                              int32_t* chunk_counts, hipStream_t s) {
+  if (chunk_tokens != 64 && chunk_tokens != 128) return DLB_ERR_BAD_ARG;
+  const dim3 grid((uint32_t)ceil_div(T, chunk_tokens)), block(1024);
   const bool a16 = aligned16(logits) && (ld_logits % 4 == 0);
-  if (E <= 64) {
-    hipLaunchKernelGGL(moe_topk_softmax_count_kernel<4>, grid, block, 0, s, logits, weights, ids, T,
-                       E, K, ld_logits, renormalize, (int)(a16 && E == 64), chunk_counts);
-  } else if (E <= 128) {
-    hipLaunchKernelGGL(moe_topk_softmax_count_kernel<8>, grid, block, 0, s, logits, weights, ids, T,
-                       E, K, ld_logits, renormalize, (int)(a16 && E == 128), chunk_counts);
-  } else {
-    hipLaunchKernelGGL(moe_topk_softmax_count_kernel<16>, grid, block, 0, s, logits, weights, ids, T,
-                       E, K, ld_logits, renormalize, (int)(a16 && E == 256), chunk_counts);
-  }
+#define DLB_LAUNCH_ROUTE_COUNT(VPL_, EFULL_)                                                     \
+  do {                                                                                           \
+    if (chunk_tokens == 64)                                                                      \
+      hipLaunchKernelGGL((moe_topk_softmax_count_kernel<VPL_, 1>), grid, block, 0, s, logits,    \
+                         weights, ids, T, E, K, ld_logits, renormalize, (int)(a16 && E == EFULL_), \
+                         chunk_counts);                                                          \
+    else                                                                                         \
+      hipLaunchKernelGGL((moe_topk_softmax_count_kernel<VPL_, 2>), grid, block, 0, s, logits,    \
+                         weights, ids, T, E, K, ld_logits, renormalize, (int)(a16 && E == EFULL_), \
+                         chunk_counts);                                                          \
+  } while (0)
+  if (E <= 64) DLB_LAUNCH_ROUTE_COUNT(4, 64);
+  else if (E <= 128) DLB_LAUNCH_ROUTE_COUNT(8, 128);
+  else DLB_LAUNCH_ROUTE_COUNT(16, 256);
+#undef DLB_LAUNCH_ROUTE_COUNT
   return launch_status();
 }
 

@@ -126,6 +126,7 @@ def test_end_to_end_config2(dev):
 @pytest.mark.parametrize("T,E,k,block", [(16384, 64, 6, 64), (1, 64, 6, 64), (127, 8, 2, 16),
                                          (128, 60, 6, 64), (129, 64, 8, 128), (333, 160, 6, 32),
                                          (5000, 256, 16, 64), (32768, 16, 4, 64), (0, 64, 6, 64),
+                                         (63, 64, 6, 64), (65, 64, 6, 64), (16385, 64, 6, 64),  # 64- / 128-token chunks
                                          (40000, 64, 6, 64)])   # the last one: the two-call path
 @pytest.mark.parametrize("renorm", [True, False])
 def test_fused_router_and_alignment_equals_the_two_calls(dev, T, E, k, block, renorm):
