@@ -87,6 +87,7 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     return sorted_ids, expert_ids, num_post
 
 
+_FUSED_PLANS = {}   # (T, E, k, block) -> (piece sizes, total words) of the result buffer
 _FUSED_MAX_TOKENS = 32768  # beyond this the fused entry point declines (DLB_ERR_UNSUPPORTED)
 
 
@@ -119,15 +120,20 @@ def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_ex
     cap = numel + E * (block_size - 1)
     nblk = max(1, -(-cap // block_size))
     lib = _lib.load()
-    ws_words = max((lib.dlb_moe_topk_softmax_align_ws_bytes(T, E) + 3) // 4, 1)
-    # one allocation of 4-byte words, carved into the results and the scratch
-    sizes = (numel, numel, cap, nblk, 1, ws_words)
-    offs, total = [], 0
-    for n in sizes:
-        offs.append(total)
-        total += (n + 3) & ~3
+    plan = _FUSED_PLANS.get((T, E, k, block_size))
+    if plan is None:
+        ws_words = max((lib.dlb_moe_topk_softmax_align_ws_bytes(T, E) + 3) // 4, 1)
+        # one allocation of 4-byte words, carved into the results and the scratch (each piece
+        # followed by the padding that keeps the next one 16-byte aligned)
+        pieces = []
+        for n in (numel, numel, cap, nblk, 1, ws_words):
+            pieces += [n, -n & 3]
+        if len(_FUSED_PLANS) > 64:
+            _FUSED_PLANS.clear()
+        plan = _FUSED_PLANS[(T, E, k, block_size)] = (pieces, sum(pieces))
+    pieces, total = plan
     buf = torch.empty((total,), dtype=torch.int32, device=dev)
-    w_raw, ids, sorted_ids, expert_ids, num_post, ws = (buf[o:o + n] for o, n in zip(offs, sizes))
+    w_raw, _, ids, _, sorted_ids, _, expert_ids, _, num_post, _, ws, _ = buf.split(pieces)
     weights = w_raw.view(torch.float32).view(T, k)
     ids = ids.view(T, k)
     with _lib.device_guard(dev):
