@@ -35,7 +35,7 @@ struct FillParams {
   int vec;                       // 1: 16-byte chunks, 0: single bytes
 };
 
-constexpr int kFillTokens = 4;  // tokens (= wavefronts) per workgroup
+constexpr int kFillTokens = 1;  // tokens (= wavefronts) per workgroup; 2 and 4 measured 1.5 % and 3.7 % slower
 
 // One wavefront per new token: it finds the sequence that owns the token with a ballot over
 // the batch, then streams the token's K and V rows into the page slot (no barriers).
