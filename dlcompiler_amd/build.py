@@ -3,10 +3,19 @@
 Run ``python -m dlcompiler_amd.build`` (cross-compiles without a GPU).  Every ``*.hip`` file
 becomes one object; objects are rebuilt only when the source or a header is newer, unless
 ``force`` is set.
+
+The compiler's per-kernel resource report (registers, scratch, spills) is collected for every
+object and written next to it.  Several kernels issue their loads through inline assembly with
+hand-counted ``s_waitcnt`` values: a register the allocator spills or copies through scratch
+memory between such a load and its wait would be read before the data has landed, and scratch
+traffic would also change the vector-memory counts the waits assume.  The build therefore fails
+when one of those kernels reports scratch memory or spilled vector registers.
 """
 from __future__ import annotations
 
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -31,7 +40,13 @@ DEVICE_FLAGS = [
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # the direct-to-LDS helpers list m0 (a reserved register) among their clobbers on purpose
+    "-Wno-inline-asm",
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# kernels whose loads and waits are issued by hand: no scratch, no spilled vector registers
+HAND_SCHEDULED = ("moe_gemm", "prefill_attn_kernel", "paged_decode_split_kernel")
 
 
 def _sources() -> list[Path]:
@@ -49,13 +64,67 @@ def _stale(target: Path, deps: list[Path]) -> bool:
     return any(d.stat().st_mtime > t for d in deps)
 
 
+_REMARK = re.compile(r"remark:\s+(.*?)\s*\[-Rpass-analysis=kernel-resource-usage\]")
+_FIELDS = {"VGPRs": "vgprs", "AGPRs": "agprs", "TotalSGPRs": "sgprs",
+           "ScratchSize [bytes/lane]": "scratch_bytes", "VGPRs Spill": "vgpr_spills",
+           "SGPRs Spill": "sgpr_spills", "Occupancy [waves/SIMD]": "occupancy",
+           "LDS Size [bytes/block]": "lds_bytes"}
+
+
+def parse_resource_remarks(stderr: str) -> dict[str, dict[str, int]]:
+    """``{mangled kernel name: {vgprs, agprs, sgprs, scratch_bytes, vgpr_spills, ...}}`` from the
+    ``-Rpass-analysis=kernel-resource-usage`` remarks of one hipcc run."""
+    kernels: dict[str, dict[str, int]] = {}
+    cur = None
+    for line in stderr.splitlines():
+        m = _REMARK.search(line)
+        if not m:
+            continue
+        key, _, val = m.group(1).partition(":")
+        key, val = key.strip(), val.strip()
+        if key == "Function Name":
+            cur = kernels.setdefault(val, {})
+        elif cur is not None and key in _FIELDS and val.lstrip("-").isdigit():
+            cur[_FIELDS[key]] = int(val)
+    return kernels
+
+
+def check_hand_scheduled(kernels: dict[str, dict[str, int]]) -> list[str]:
+    """Names (with the offending figures) of hand-scheduled kernels that use scratch or spill."""
+    bad = []
+    for name, r in kernels.items():
+        if any(tag in name for tag in HAND_SCHEDULED):
+            if r.get("scratch_bytes", 0) or r.get("vgpr_spills", 0):
+                bad.append(f"{name}: scratch {r.get('scratch_bytes', 0)} B/lane, "
+                           f"{r.get('vgpr_spills', 0)} spilled VGPRs")
+    return bad
+
+
 def _compile_one(src: Path, obj: Path, verbose: bool) -> None:
     cmd = [HIPCC, *DEVICE_FLAGS, f"-I{INCLUDE_DIR}", "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    noise = ("is not a recognized feature for this target", "-Rpass-analysis=kernel-resource-usage")
+    lines = proc.stderr.splitlines()
+    keep, skip = [], 0
+    for l in lines:
+        if any(n in l for n in noise):
+            skip = 2 if "-Rpass-analysis" in l and "Function Name" in l else 0
+            continue
+        if skip and (l.lstrip().startswith(("|", "^")) or re.match(r"\s*\d+ \|", l)):
+            skip -= 1  # the source excerpt printed under a remark
+            continue
+        keep.append(l)
+    err = "\n".join(keep)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{err}")
+    kernels = parse_resource_remarks(proc.stderr)
+    report = obj.with_suffix(".resources.json")
+    report.write_text(json.dumps(kernels, indent=1, sort_keys=True))
+    bad = check_hand_scheduled(kernels)
+    if bad:
+        obj.unlink(missing_ok=True)
+        raise RuntimeError(f"{src.name}: hand-scheduled kernels must not spill or use scratch:\n  "
+                           + "\n  ".join(bad))
     if verbose and err.strip():
         print(err, file=sys.stderr)
 
@@ -82,6 +151,14 @@ def build_library(force: bool = False, verbose: bool = False, jobs: int | None =
         if proc.returncode != 0:
             raise RuntimeError(f"link failed:\n{proc.stderr}")
     return LIB_PATH
+
+
+def kernel_resources() -> dict[str, dict[str, int]]:
+    """The resource reports of the last build of every object, merged."""
+    merged: dict[str, dict[str, int]] = {}
+    for rep in sorted(OBJ_DIR.glob("*.resources.json")):
+        merged.update(json.loads(rep.read_text()))
+    return merged
 
 
 if __name__ == "__main__":

@@ -128,11 +128,13 @@ __device__ __forceinline__ unsigned int lds_addr(const void* p) {
 // does not see it, so the caller waits for it explicitly (s_waitcnt vmcnt) before the barrier
 // that publishes the data.  Waits the compiler inserts for its own loads stay correct: an
 // unseen load that is older completes first, one that is younger only makes the wait longer.
+// The helpers write m0 and say so in their clobber lists, so the compiler never keeps a live
+// value of its own (an LDS-direct or indexed-register base) in m0 across one of them.
 __device__ __forceinline__ void dma16_global_to_lds(const void* gsrc, unsigned int lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base))
-               : "memory");
+               : "memory", "m0");
 }
 
 // same copy, addressed as a wave-uniform 64-bit base (scalar registers) plus a 32-bit lane offset
@@ -141,7 +143,7 @@ __device__ __forceinline__ void dma16_global_to_lds(const void* sbase, unsigned 
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane((int)lds_base))
-               : "memory");
+               : "memory", "m0");
 }
 
 // the 4-byte form: lane l's dword lands at lds_base + 4 * l
@@ -149,7 +151,7 @@ __device__ __forceinline__ void dma4_global_to_lds(const void* gsrc, unsigned in
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                :
                : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base))
-               : "memory");
+               : "memory", "m0");
 }
 
 // the 4-byte form restricted to the lanes of `lane_mask` (a compile-time constant); the other
@@ -161,7 +163,7 @@ __device__ __forceinline__ void dma4_global_to_lds_masked(const void* gsrc, unsi
                "global_load_lds_dword %1, off\n\ts_mov_b64 exec, %0"
                : "=&s"(saved)
                : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "n"(lane_mask)
-               : "memory");
+               : "memory", "m0");
 }
 
 // ds_read_b64_tr_b16: every lane passes the address of four consecutive 16-bit elements; in
