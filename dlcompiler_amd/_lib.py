@@ -28,6 +28,9 @@ SIGNATURES = {
     "dlb_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                          c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                          c_size_t, c_void_p]),
+    "dlb_moe_align_block_size_static_max_numel": (c_int64, []),
+    "dlb_moe_align_block_size_static": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+                                                c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "dlb_moe_topk_softmax_align_ws_bytes": (c_size_t, [c_int64, c_int]),
     "dlb_moe_topk_softmax_align_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
                                                c_int64, c_int, c_int, c_void_p, c_int64, c_void_p,

@@ -16,6 +16,8 @@
 //              start[chunk][e] + (number of earlier i' in the chunk with the same e), the rank
 //              coming from wave ballots, which makes the sort stable (ascending i per expert).
 // Integer work only; no float or order-dependent atomics, so the output is bit-reproducible.
+#include <mutex>
+
 #include "common.h"
 
 namespace dlb {
@@ -333,12 +335,13 @@ extern "C" size_t dlb_moe_align_ws_bytes(int64_t numel, int E) {
   return (size_t)dlb::num_chunks(numel) * (size_t)E * sizeof(int32_t);
 }
 
-extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int block,
-                                        int32_t* sorted_ids, int64_t sorted_cap,
-                                        int32_t* expert_ids, int64_t expert_ids_cap,
-                                        int32_t* counts, int32_t* num_post_pad, void* ws,
-                                        size_t ws_bytes, void* stream) {
-  using namespace dlb;
+namespace dlb {
+namespace {
+
+// argument checks shared by the two alignment entry points (everything but the scratch)
+int check_align_args(const int32_t* topk_ids, int64_t numel, int E, int block,
+                     const int32_t* sorted_ids, int64_t sorted_cap, const int32_t* expert_ids,
+                     int64_t expert_ids_cap, const int32_t* num_post_pad) {
   if (numel < 0 || E < 1 || block < 1) return DLB_ERR_BAD_ARG;
   if (E > kMaxE) return DLB_ERR_UNSUPPORTED;
   if (numel + (int64_t)E * block >= (int64_t)0x7fffffff) return DLB_ERR_UNSUPPORTED;
@@ -346,10 +349,15 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
     return DLB_ERR_BAD_ARG;
   if (sorted_cap < numel + (int64_t)E * (block - 1)) return DLB_ERR_BAD_ARG;
   if (expert_ids_cap < ceil_div(sorted_cap, block)) return DLB_ERR_BAD_ARG;
-  if (!ws || ws_bytes < dlb_moe_align_ws_bytes(numel, E)) return DLB_ERR_WORKSPACE;
-  hipStream_t s = (hipStream_t)stream;
+  return DLB_OK;
+}
+
+// the launches of the alignment; chunk_counts holds num_chunks(numel) x E int32, every word of
+// which the counting pass overwrites before anything reads it (nothing has to start at zero)
+int launch_align(const int32_t* topk_ids, int64_t numel, int E, int block, int32_t* sorted_ids,
+                 int64_t sorted_cap, int32_t* expert_ids, int64_t expert_ids_cap, int32_t* counts,
+                 int32_t* num_post_pad, int32_t* chunk_counts, hipStream_t s) {
   const int64_t chunks = num_chunks(numel);
-  int32_t* chunk_counts = (int32_t*)ws;
   hipLaunchKernelGGL(align_count_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
                      numel, E, chunk_counts);
   if (chunks <= kFusedChunks) {
@@ -366,6 +374,74 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
     hipLaunchKernelGGL(align_place_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
                        numel, E, chunk_counts, sorted_ids);
   return launch_status();
+}
+
+// ---- scratch of the entry point that allocates nothing --------------------------------------
+// The per-chunk count table of up to kStaticChunks chunks x kMaxE experts (256 KB) lives in a
+// file-scope device array: every GPU the library runs on holds one copy of it until the process
+// ends.  In host code the array's name is only a handle, not a device address; the address on
+// the current device comes from hipGetSymbolAddress, once per device, and is what the kernels
+// receive.
+constexpr int kStaticChunks = kFusedChunks;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) int32_t scratch[kStaticChunks * kMaxE];
+
+std::mutex scratch_mutex;
+int32_t* scratch_ptr[kMaxDevices];  // per device, filled on the first call made on that device
+
+int static_scratch(int32_t** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return DLB_ERR_LAUNCH;
+  std::lock_guard<std::mutex> guard(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return DLB_ERR_LAUNCH;
+    }
+    scratch_ptr[dev] = (int32_t*)ptr;
+  }
+  *out = scratch_ptr[dev];
+  return DLB_OK;
+}
+
+}  // namespace
+}  // namespace dlb
+
+extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int block,
+                                        int32_t* sorted_ids, int64_t sorted_cap,
+                                        int32_t* expert_ids, int64_t expert_ids_cap,
+                                        int32_t* counts, int32_t* num_post_pad, void* ws,
+                                        size_t ws_bytes, void* stream) {
+  using namespace dlb;
+  const int st = check_align_args(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                                  expert_ids_cap, num_post_pad);
+  if (st != DLB_OK) return st;
+  if (!ws || ws_bytes < dlb_moe_align_ws_bytes(numel, E)) return DLB_ERR_WORKSPACE;
+  return launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                      expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream);
+}
+
+extern "C" int64_t dlb_moe_align_block_size_static_max_numel(void) {
+  return (int64_t)dlb::kStaticChunks * dlb::kChunk;
+}
+
+extern "C" int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int E,
+                                               int block, int32_t* sorted_ids, int64_t sorted_cap,
+                                               int32_t* expert_ids, int64_t expert_ids_cap,
+                                               int32_t* counts, int32_t* num_post_pad,
+                                               void* stream) {
+  using namespace dlb;
+  const int st = check_align_args(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                                  expert_ids_cap, num_post_pad);
+  if (st != DLB_OK) return st;
+  // the static table holds kStaticChunks chunks: larger inputs must bring their own workspace
+  if (numel > dlb_moe_align_block_size_static_max_numel()) return DLB_ERR_WORKSPACE;
+  int32_t* chunk_counts = nullptr;
+  const int sp = static_scratch(&chunk_counts);
+  if (sp != DLB_OK) return sp;
+  return launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                      expert_ids_cap, counts, num_post_pad, chunk_counts, (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -91,6 +91,23 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
                              void* ws, size_t ws_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * dlb_moe_align_block_size without a workspace argument and without any allocation: same
+ * arguments, same results bit for bit.  It has no counterpart in the reference; it exists for
+ * callers that cannot allocate device memory around the call (code under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  The scratch (the per-chunk count
+ * table) is a 256 KB array in the library's device image, one copy per GPU, held until the
+ * process ends.  Limit: numel <= dlb_moe_align_block_size_static_max_numel() (524288 routing
+ * slots); more returns DLB_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls
+ * that overlap on one GPU (different streams) race; calls on one stream are ordered.  Nothing
+ * in the array has to be cleared between calls.
+ * ---------------------------------------------------------------------------------------- */
+int64_t dlb_moe_align_block_size_static_max_numel(void);
+int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int E, int block,
+                                    int32_t* sorted_ids, int64_t sorted_cap,
+                                    int32_t* expert_ids, int64_t expert_ids_cap, int32_t* counts,
+                                    int32_t* num_post_pad, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Router and alignment in one call (two launches instead of three): the outputs of
  * dlb_moe_topk_softmax_f32 followed by dlb_moe_align_block_size on its ids, bit for bit.
  * The same reference lines as the two calls above: the router of
