@@ -45,10 +45,12 @@ SIGNATURES = {
                                + [c_float, c_int, c_float, c_int, c_void_p]),
     "dlb_per_token_group_quant_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                               c_int64, c_int64, c_int64, c_int, c_void_p]),
-    "dlb_moe_gemm_fp8_gate_up": (c_int, [c_void_p] * 6 + [c_int] * 9 + [c_void_p] * 3),
-    "dlb_moe_gemm_fp8_down": (c_int, [c_void_p] * 7 + [c_int] * 9 + [c_void_p, c_int, c_void_p]),
-    "dlb_moe_gemm_16bit_gate_up": (c_int, [c_void_p] * 4 + [c_int] * 9 + [c_void_p, c_int, c_void_p]),
-    "dlb_moe_gemm_16bit_down": (c_int, [c_void_p] * 5 + [c_int] * 9 + [c_void_p, c_int, c_void_p]),
+    "dlb_moe_gemm_fp8_gate_up": (c_int, [c_void_p] * 6 + [c_int] * 10 + [c_void_p] * 3),
+    "dlb_moe_gemm_fp8_down": (c_int, [c_void_p] * 6 + [c_int, c_void_p] + [c_int] * 9
+                              + [c_void_p, c_int, c_void_p]),
+    "dlb_moe_gemm_16bit_gate_up": (c_int, [c_void_p] * 4 + [c_int] * 10 + [c_void_p, c_int, c_void_p]),
+    "dlb_moe_gemm_16bit_down": (c_int, [c_void_p] * 4 + [c_int, c_void_p] + [c_int] * 9
+                                + [c_void_p, c_int, c_void_p]),
     "dlb_fill_kv_cache": (c_int, [c_void_p] * 8 + [c_int64] + [c_int] * 7 + [c_int64] * 11
                           + [c_void_p]),
     "dlb_rms_norm": (c_int, [c_void_p] * 5 + [c_int64, c_int] + [c_int64] * 4

@@ -107,6 +107,19 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// inclusive prefix sum over the 64 lanes of a wave with DPP moves only (shifts inside each row
+// of 16 lanes, then the row totals broadcast to the rows after them): no LDS round trips and no
+// per-lane address registers, which a shuffle-based scan keeps live across the whole kernel
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
+  return v;
+}
+
 // a pointer the caller knows to be wave-uniform, moved into scalar registers
 __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
   const uint64_t v = (uint64_t)(uintptr_t)p;
@@ -162,7 +175,7 @@ __device__ __forceinline__ void dma4_global_to_lds_masked(const void* gsrc, unsi
   asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
                "global_load_lds_dword %1, off\n\ts_mov_b64 exec, %0"
                : "=&s"(saved)
-               : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "n"(lane_mask)
+               : "v"(gsrc), "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "s"(lane_mask)
                : "memory", "m0");
 }
 
@@ -174,6 +187,19 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const void* p) {
   typedef __attribute__((ext_vector_type(4))) short s16x4;
   typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
   return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p));
+}
+
+// the masked 4-byte form addressed as a wave-uniform 64-bit base plus a 32-bit lane offset
+template <unsigned long long lane_mask>
+__device__ __forceinline__ void dma4_global_to_lds_masked(const void* sbase, unsigned int voff,
+                                                          unsigned int lds_base) {
+  unsigned long long saved;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+               "global_load_lds_dword %1, %2\n\ts_mov_b64 exec, %0"
+               : "=&s"(saved)
+               : "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane((int)lds_base)),
+                 "s"(lane_mask)
+               : "memory", "m0");
 }
 
 // max of a value and its partner 32 lanes away (v_permlane32_swap: a register-file exchange,

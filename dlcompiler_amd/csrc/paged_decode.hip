@@ -81,19 +81,6 @@ struct Mma16<DLB_DTYPE_F16> {
   }
 };
 
-// inclusive prefix sum over the 64 lanes of a wave with DPP moves only (shifts inside each row
-// of 16 lanes, then the row totals broadcast to the rows after them): no LDS round trips and no
-// per-lane address registers, which a shuffle-based scan keeps live across the whole kernel
-__device__ __forceinline__ int wave_inclusive_scan(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
-  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
-  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
-  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
-  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
-  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
-  return v;
-}
-
 constexpr int kTile = 64;          // keys per iteration
 constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
 

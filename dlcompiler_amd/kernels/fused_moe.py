@@ -12,19 +12,9 @@ import torch
 from .. import _lib
 from .moe_gating import moe_align_block_size
 
-import os
-
-_BLOCK_OVERRIDE = int(os.environ.get("DLB_MOE_BLOCK", "0"))  # 64 / 128 force a tile height
-
-
-def _align_block(weights_shuffled: bool) -> int:
-    """Rows per grouped-GEMM workgroup tile = alignment block of the routing.  Row-major
-    weights (the reference layout) run fastest on the 128-row kernel, which stages them through
-    LDS a full cache line per row; operand-order weights on the 64-row kernel, which streams
-    them straight into MFMA operand registers."""
-    if _BLOCK_OVERRIDE in (64, 128):
-        return _BLOCK_OVERRIDE
-    return 64 if weights_shuffled else 128
+# rows per grouped-GEMM workgroup tile = alignment block of the routing; tiles skip 32-row groups
+# that hold padding only, so the matrix work follows the routed rows in steps of 32
+_BLOCK_M = 128
 
 
 def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
@@ -92,36 +82,35 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
                   expert_offset: int = 0,
                   num_experts: int = None,
                   renormalize: bool = False,
-                  weights_shuffled: bool = False,
-                  _stage_hook=None) -> torch.Tensor:
+                  weights_shuffled: bool = False) -> torch.Tensor:
     """fp8 MoE MLP: per-token-group quant -> gate_up grouped GEMM (+SiLU-and-mul, re-quant)
     -> down grouped GEMM (x routing weight) -> sum over the top-k slots.
 
-    ``hidden_states`` [T, H] bf16/f16; ``w1_q`` [E, 2I, H] / ``w2_q`` [E, H, I]
+    ``hidden_states`` [T, H] bf16/f16; ``w1_q`` [E, 2I, H] / ``w2_q`` [E, O, I]
     float8_e4m3fn with fp32 scales per 128x128 block (``w1_s`` [E, 2I/128, H/128],
-    ``w2_s`` [E, H/128, I/128]); ``topk_weights``/``topk_ids`` [T, topk].  ``E`` is the
-    number of local experts, holding global experts ``expert_offset .. expert_offset + E``;
-    ``num_experts`` the global count (defaults to ``E``), as in the reference.
-    ``weights_shuffled=True`` says ``w1_q``/``w2_q`` went through
+    ``w2_s`` [E, O/128, I/128]); ``topk_weights``/``topk_ids`` [T, topk].  The output is
+    [T, O]; as in the reference its width comes from ``w2`` (fused_moe.py:354-357) and is
+    normally H.  ``E`` is the number of local experts, holding global experts
+    ``expert_offset .. expert_offset + E``; ``num_experts`` the global count (defaults to
+    ``E``), as in the reference.  ``weights_shuffled=True`` says ``w1_q``/``w2_q`` went through
     :func:`shuffle_moe_weight_fp8` (same shapes, operand-order bytes) -- the fast path.
-    ``_stage_hook(name)`` is called before each stage (profiling aid).
     """
-    hook = _stage_hook or (lambda name: None)
     _lib.require_cuda(hidden_states, w1_q, w1_s, w2_q, w2_s, topk_weights, topk_ids)
     assert hidden_states.dim() == 2 and topk_ids.shape == topk_weights.shape
     T, H = hidden_states.shape
     E, N2, H1 = w1_q.shape
     I = N2 // 2
-    assert H1 == H and w2_q.shape == (E, H, I) and topk_ids.shape == (T, topk)
+    O = w2_q.shape[1]
+    assert H1 == H and w2_q.shape == (E, O, I) and topk_ids.shape == (T, topk)
     assert w1_q.dtype == torch.float8_e4m3fn and w2_q.dtype == torch.float8_e4m3fn
     assert w1_q.is_contiguous() and w2_q.is_contiguous()
-    assert w1_s.shape == (E, N2 // 128, H // 128) and w2_s.shape == (E, H // 128, I // 128)
+    assert w1_s.shape == (E, N2 // 128, H // 128) and w2_s.shape == (E, O // 128, I // 128)
     if num_experts is None:
         num_experts = E
     dev = hidden_states.device
     dt = hidden_states.dtype
     if T == 0:
-        return hidden_states.new_empty((0, H))
+        return hidden_states.new_empty((0, O))
 
     if renormalize:
         topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
@@ -129,44 +118,39 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     w1_s = w1_s.to(torch.float32).contiguous()
     w2_s = w2_s.to(torch.float32).contiguous()
 
-    hook("align")
-    block = _align_block(weights_shuffled)
-    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, block, num_experts)
-    num_mblocks = expert_ids.numel()
-    hook("quant")
+    block = _BLOCK_M
+    sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
+                                                    return_counts=True)
+    num_mblocks = -(-sorted_ids.numel() // block)
     xq, xs = per_token_group_quant_fp8(hidden_states)
-    hook("alloc")
 
+    # one allocation for the intermediates: fp8 rows + their scales (fp32) + the slot outputs
     rows = num_mblocks * block
+    full = (expert_offset == 0 and num_experts == E)
     hq = torch.empty((rows, I), dtype=torch.float8_e4m3fn, device=dev)
     hs = torch.empty((rows, I // 128), dtype=torch.float32, device=dev)
-    full = (expert_offset == 0 and num_experts == E)
-    slots = (torch.empty if full else torch.zeros)((T * topk, H), dtype=dt, device=dev)
-    out = torch.empty((T, H), dtype=dt, device=dev)
+    slots = (torch.empty if full else torch.zeros)((T * topk, O), dtype=dt, device=dev)
+    out = torch.empty((T, O), dtype=dt, device=dev)
 
     lib = _lib.load()
     stream = _lib.current_stream_ptr(dev)
     with _lib.device_guard(dev):
-        hook("gate_up")
         st = lib.dlb_moe_gemm_fp8_gate_up(xq.data_ptr(), xs.data_ptr(), w1_q.data_ptr(),
                                           w1_s.data_ptr(), sorted_ids.data_ptr(),
-                                          expert_ids.data_ptr(), num_mblocks, block, T, topk,
-                                          H, I, expert_offset, E, int(weights_shuffled),
+                                          counts.data_ptr(), num_experts, num_mblocks, block, T,
+                                          topk, H, I, expert_offset, E, int(weights_shuffled),
                                           hq.data_ptr(), hs.data_ptr(), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_gate_up")
-        hook("down")
         st = lib.dlb_moe_gemm_fp8_down(hq.data_ptr(), hs.data_ptr(), w2_q.data_ptr(),
                                        w2_s.data_ptr(), sorted_ids.data_ptr(),
-                                       expert_ids.data_ptr(), topk_weights.data_ptr(),
-                                       num_mblocks, block, T, topk, H, I, expert_offset, E,
+                                       counts.data_ptr(), num_experts, topk_weights.data_ptr(),
+                                       num_mblocks, block, T, topk, O, I, expert_offset, E,
                                        int(weights_shuffled),
                                        slots.data_ptr(), _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_gemm_fp8_down")
-        hook("topk_sum")
-        st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), T, topk, H,
+        st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), T, topk, O,
                                   _lib.torch_dtype_code(dt), stream)
         _lib.check(st, "dlb_moe_topk_sum")
-        hook(None)
     return out
 
 
@@ -191,14 +175,15 @@ def fused_moe(hidden_states: torch.Tensor,
     E, N, _ = w1.shape
     H = hidden_states.size(1)
     I = N // 2
-    assert w1.shape == (E, 2 * I, H) and w2.shape == (E, H, I)
+    O = w2.shape[1]  # output width, taken from w2 as in the reference (fused_moe.py:354-357)
+    assert w1.shape == (E, 2 * I, H) and w2.shape == (E, O, I)
     assert hidden_states.dtype == w1.dtype == w2.dtype
     assert w1.is_contiguous() and w2.is_contiguous()
     if num_experts is None:
         num_experts = E
     dev, dt = hidden_states.device, hidden_states.dtype
     if M == 0:
-        return hidden_states.new_empty((0, H))
+        return hidden_states.new_empty((0, O))
     if hidden_states.stride(1) != 1 or hidden_states.stride(0) != H:
         hidden_states = hidden_states.contiguous()
 
@@ -206,28 +191,30 @@ def fused_moe(hidden_states: torch.Tensor,
         topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
     topk_weights = topk_weights.to(torch.float32).contiguous()
 
-    block = _align_block(weights_shuffled)
-    sorted_ids, expert_ids, _ = moe_align_block_size(topk_ids, block, num_experts)
-    num_mblocks = expert_ids.numel()
+    block = _BLOCK_M
+    sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
+                                                    return_counts=True)
+    num_mblocks = -(-sorted_ids.numel() // block)
     act = torch.empty((num_mblocks * block, I), dtype=dt, device=dev)
     full = (expert_offset == 0 and num_experts == E)
-    slots = (torch.empty if full else torch.zeros)((M * topk, H), dtype=dt, device=dev)
-    out = torch.empty((M, H), dtype=dt, device=dev)
+    slots = (torch.empty if full else torch.zeros)((M * topk, O), dtype=dt, device=dev)
+    out = torch.empty((M, O), dtype=dt, device=dev)
     lib = _lib.load()
     code = _lib.torch_dtype_code(dt)
     stream = _lib.current_stream_ptr(dev)
     with _lib.device_guard(dev):
         st = lib.dlb_moe_gemm_16bit_gate_up(hidden_states.data_ptr(), w1.data_ptr(),
-                                            sorted_ids.data_ptr(), expert_ids.data_ptr(),
-                                            num_mblocks, block, M, topk, H, I,
+                                            sorted_ids.data_ptr(), counts.data_ptr(),
+                                            num_experts, num_mblocks, block, M, topk, H, I,
                                             expert_offset, E, int(weights_shuffled),
                                             act.data_ptr(), code, stream)
         _lib.check(st, "dlb_moe_gemm_16bit_gate_up")
         st = lib.dlb_moe_gemm_16bit_down(act.data_ptr(), w2.data_ptr(), sorted_ids.data_ptr(),
-                                         expert_ids.data_ptr(), topk_weights.data_ptr(),
-                                         num_mblocks, block, M, topk, H, I, expert_offset,
-                                         E, int(weights_shuffled), slots.data_ptr(), code, stream)
+                                         counts.data_ptr(), num_experts,
+                                         topk_weights.data_ptr(), num_mblocks, block, M, topk,
+                                         O, I, expert_offset, E, int(weights_shuffled),
+                                         slots.data_ptr(), code, stream)
         _lib.check(st, "dlb_moe_gemm_16bit_down")
-        st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), M, topk, H, code, stream)
+        st = lib.dlb_moe_topk_sum(slots.data_ptr(), out.data_ptr(), M, topk, O, code, stream)
         _lib.check(st, "dlb_moe_topk_sum")
     return out

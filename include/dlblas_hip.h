@@ -219,19 +219,21 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
 /* gate_up grouped GEMM + SiLU-and-mul + re-quantisation.
  *   xq [num_tokens, H] fp8, xs [num_tokens, H/128]
  *   w1q [num_local_experts, 2I, H] fp8 (gate rows first), w1s [num_local_experts, 2I/128, H/128]
- *   sorted_ids [num_mblocks * block_m], expert_ids [num_mblocks]: output of
- *     dlb_moe_align_block_size with block = block_m, block_m in {64, 128} = rows per
- *     workgroup tile (flat slot = token * topk + j, sentinel
- *     num_tokens * topk, expert -1 for unused blocks); blocks whose expert lies outside
- *     [expert_offset, expert_offset + num_local_experts) are skipped
+ *   sorted_ids [num_mblocks * block_m] and expert_counts [num_experts]: the sorted slot list and
+ *     the per-expert counts written by dlb_moe_align_block_size with block = block_m over all
+ *     num_experts (global) experts; block_m in {64, 128} = rows per workgroup tile; flat slot =
+ *     token * topk + j, sentinel num_tokens * topk.  num_mblocks = capacity of sorted_ids in
+ *     blocks (>= sum over experts of ceil(count / block_m)).  Expert e's blocks start at block
+ *     sum_{e' < e} ceil(count[e'] / block_m); blocks of experts outside
+ *     [expert_offset, expert_offset + num_local_experts) are skipped.  num_experts <= 256.
  *   hq [num_mblocks * block_m, I] fp8 and hs [num_mblocks * block_m, I/128]: row r holds
- *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r
- * H % 128 == 0, I % 128 == 0.
- * block_m selects the kernel: 64 = four-wave tiles of 64 rows, weights streamed straight into
- * operand registers (fastest with w_layout 1); 128 = eight-wave tiles of 128 rows x 256
- * columns with both operands staged by direct-to-LDS loads (reads row-major weights, w_layout
- * 0, at full efficiency).  Outputs are stored 16 bytes at a time: hq, out and the 16-bit act
- * must be 16-byte aligned; other alignments return DLB_ERR_UNSUPPORTED.
+ *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r (rows of
+ *     32-row groups that hold padding only are not written)
+ * H % 128 == 0, I % 128 == 0; scales must be positive (values below 1e-30 count as 1e-30).
+ * One kernel serves both tile heights and both weight layouts: four-wave tiles of block_m rows
+ * x 256 columns, weights streamed straight into operand registers, activations staged in LDS.
+ * Outputs are stored 16 bytes at a time: hq, out and the 16-bit act must be 16-byte aligned;
+ * other alignments return DLB_ERR_UNSUPPORTED.
  * w_layout selects how the fp8 weight bytes of both GEMMs are stored:
  *   0  row-major [E, N, K] (the reference's w1/w2 layout);
  *   1  MFMA-operand order, a one-time re-arrangement done when the weights are loaded: for
@@ -240,18 +242,20 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
  *      W[e][16 nb + l % 16][128 kc + 64 h + 16 (l / 16) .. + 16].  Same bytes, same scales;
  *      every operand load becomes one contiguous 1 KB access. */
 int dlb_moe_gemm_fp8_gate_up(const void* xq, const float* xs, const void* w1q, const float* w1s,
-                             const int32_t* sorted_ids, const int32_t* expert_ids,
-                             int num_mblocks, int block_m, int num_tokens, int topk, int H, int I,
-                             int expert_offset, int num_local_experts, int w_layout, void* hq,
-                             float* hs, void* stream);
+                             const int32_t* sorted_ids, const int32_t* expert_counts,
+                             int num_experts, int num_mblocks, int block_m, int num_tokens,
+                             int topk, int H, int I, int expert_offset, int num_local_experts,
+                             int w_layout, void* hq, float* hs, void* stream);
 
 /* down grouped GEMM: out[slot, :] = (h_r W_down^T) * topk_weights[slot] for every real slot
  * (pad rows are skipped), out [num_tokens * topk, H] bf16/f16;
- * w2q [num_local_experts, H, I] fp8, w2s [num_local_experts, H/128, I/128]. */
+ * w2q [num_local_experts, H, I] fp8, w2s [num_local_experts, H/128, I/128].  H is the output
+ * width of this GEMM (the reference takes it from w2.shape[1], kernels/fused_moe.py:354-357): it
+ * need not equal the H of the gate_up call. */
 int dlb_moe_gemm_fp8_down(const void* hq, const float* hs, const void* w2q, const float* w2s,
-                          const int32_t* sorted_ids, const int32_t* expert_ids,
-                          const float* topk_weights, int num_mblocks, int block_m,
-                          int num_tokens, int topk, int H, int I, int expert_offset,
+                          const int32_t* sorted_ids, const int32_t* expert_counts,
+                          int num_experts, const float* topk_weights, int num_mblocks,
+                          int block_m, int num_tokens, int topk, int H, int I, int expert_offset,
                           int num_local_experts, int w_layout, void* out, int out_dtype,
                           void* stream);
 
@@ -263,7 +267,7 @@ int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk, in
 /* ------------------------------------------------------------------------------------------
  * Unquantised (bf16/f16) fused MoE: the reference's own fused_moe pipeline,
  * kernels/fused_moe.py:82-235 (grouped GEMM kernel + launcher) and :334-373 (the two calls).
- * Same routing inputs, tile height and weight layouts as the fp8 GEMMs above (w_layout 1 is
+ * Same routing inputs (sorted_ids, expert_counts), tile height and weight layouts as the fp8 GEMMs above (w_layout 1 is
  * the same byte re-arrangement applied to the 2-byte elements: 128-byte chunks = 64 elements).
  *   gate_up: act[r, :] = round(silu(round(x_t W_gate^T)) * round(x_t W_up^T)) for the slot at
  *            sorted position r -- the rounding points of the reference (GEMM result stored in
@@ -273,15 +277,16 @@ int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk, in
  * Follow with dlb_moe_topk_sum.
  * ---------------------------------------------------------------------------------------- */
 int dlb_moe_gemm_16bit_gate_up(const void* x, const void* w1, const int32_t* sorted_ids,
-                               const int32_t* expert_ids, int num_mblocks, int block_m,
-                               int num_tokens, int topk, int H, int I, int expert_offset,
-                               int num_local_experts, int w_layout, void* act, int dtype,
-                               void* stream);
+                               const int32_t* expert_counts, int num_experts, int num_mblocks,
+                               int block_m, int num_tokens, int topk, int H, int I,
+                               int expert_offset, int num_local_experts, int w_layout, void* act,
+                               int dtype, void* stream);
 int dlb_moe_gemm_16bit_down(const void* act, const void* w2, const int32_t* sorted_ids,
-                            const int32_t* expert_ids, const float* topk_weights,
-                            int num_mblocks, int block_m, int num_tokens, int topk, int H, int I,
-                            int expert_offset, int num_local_experts, int w_layout, void* out,
-                            int dtype, void* stream);
+                            const int32_t* expert_counts, int num_experts,
+                            const float* topk_weights, int num_mblocks, int block_m,
+                            int num_tokens, int topk, int H, int I, int expert_offset,
+                            int num_local_experts, int w_layout, void* out, int dtype,
+                            void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Decoder-layer helpers around the attention / MoE kernels (memory-bound).

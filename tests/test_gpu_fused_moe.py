@@ -56,8 +56,8 @@ def test_fused_moe_parity(dev, T, H, I, E, k, dtype, monkeypatch):
         assert err < 5e-3
 
     check(fm.fused_moe(*args, k, renormalize=True))     # default tile height for row-major weights
-    for block in (64, 128):                              # both kernels, both weight layouts
-        monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+    for block in (64, 128):                              # both tile heights, both weight layouts
+        monkeypatch.setattr(fm, "_BLOCK_M", block)
         out = fm.fused_moe(*args, k, renormalize=True)
         check(out)
         out2 = fm.fused_moe(args[0], fm.shuffle_moe_weight(args[1]), fm.shuffle_moe_weight(args[2]),

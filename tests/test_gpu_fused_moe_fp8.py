@@ -61,13 +61,12 @@ def test_fused_moe_fp8_parity(dev, T, H, I, E, k, dtype, monkeypatch):
     x, w1q, w1s, w2q, w2s, tw, ids = _inputs(T, H, I, E, k, 1, dtype)
     ref = ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids)
     d = [t.to(dev) for t in (x, w1q, w1s, w2q, w2s, tw, ids)]
-    # default choice of tile height: 128-row kernel for row-major weights, 64-row for shuffled
     out = fm.fused_moe_fp8(*d, k)
     assert out.shape == (T, H) and out.dtype == dtype
     _check(out.cpu(), ref)
     sh = fm.shuffle_moe_weight_fp8
-    for block in (64, 128):                      # both kernels, both weight layouts
-        monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+    for block in (64, 128):                      # both tile heights, both weight layouts
+        monkeypatch.setattr(fm, "_BLOCK_M", block)
         plain = fm.fused_moe_fp8(*d, k)
         _check(plain.cpu(), ref)
         # operand-order weight storage: same bytes re-arranged, so the result is bit-identical
@@ -178,8 +177,8 @@ def test_config5_full(dev):
 
 @pytest.mark.parametrize("block", [64, 128])
 def test_fused_moe_fp8_repeats_bit_identically(dev, block, monkeypatch):
-    """Config-size run, repeated: the kernels issue their loads by hand with explicit waits, so a
-    missing wait would show as run-to-run differences on a busy chip."""
+    """Config-size run, repeated: the kernel issues its LDS copies by hand with explicit waits, so
+    a missing wait would show as run-to-run differences on a busy chip."""
     from dlcompiler_amd.kernels import fused_moe as fm
 
     T, H, I, E, k = 4096, 2048, 1408, 64, 6
@@ -191,7 +190,7 @@ def test_fused_moe_fp8_repeats_bit_identically(dev, block, monkeypatch):
     w2s = (torch.rand((E, H // 128, I // 128), generator=g) * 0.02 + 0.01).to(dev)
     tw, ids = torch.topk(torch.softmax(torch.randn((T, E), generator=g), -1), k)
     tw, ids = tw.to(dev), ids.int().to(dev)
-    monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+    monkeypatch.setattr(fm, "_BLOCK_M", block)
     for shuffled in (False, True):
         a = fm.shuffle_moe_weight_fp8(w1q) if shuffled else w1q
         b = fm.shuffle_moe_weight_fp8(w2q) if shuffled else w2q

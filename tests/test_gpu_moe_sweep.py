@@ -45,7 +45,7 @@ def test_fused_moe_sweep(dev, seed, monkeypatch):
     ref16 = ofm.fused_moe(x, w1h, w2h, tw, ids)
     d16 = [t.to(dev) for t in (x, w1h, w2h, tw, ids)]
     for block in (64, 128):
-        monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", block)
+        monkeypatch.setattr(fm, "_BLOCK_M", block)
         _check(fm.fused_moe_fp8(*d8, k).cpu(), ref8, 3e-2)
         shuf = fm.fused_moe_fp8(d8[0], fm.shuffle_moe_weight_fp8(d8[1]), d8[2],
                                 fm.shuffle_moe_weight_fp8(d8[3]), d8[4], d8[5], d8[6], k,
@@ -55,7 +55,7 @@ def test_fused_moe_sweep(dev, seed, monkeypatch):
 
     # an expert shard: experts [off, off + n) only, the other slots contribute nothing
     if E >= 3:
-        monkeypatch.setattr(fm, "_BLOCK_OVERRIDE", 0)
+        monkeypatch.setattr(fm, "_BLOCK_M", 128)
         off, n = 1, E - 2
         out = fm.fused_moe_fp8(d8[0], d8[1][off:off + n], d8[2][off:off + n], d8[3][off:off + n],
                                d8[4][off:off + n], d8[5], d8[6], k, expert_offset=off, num_experts=E)
