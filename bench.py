@@ -12,13 +12,16 @@ A "step" is one call of an operator's public entry point on one batch.  The top-
 the fp8 fused MoE); `workloads` carries the same figures for every configuration.
 
 For each workload:
-  value      algorithmic work / wall time of K back-to-back steps (events on the launch stream)
-  roofline   the dominant kernel: algorithmic bytes (or FLOPs) per launch / its average launch
-             duration, measured with events bracketing that kernel inside the timed loop;
-             `traffic` (HBM bytes per launch from rocprofv3 --pmc) is read from
-             profiles/hbm_traffic.json when a measurement has been committed, else null
+  value      algorithmic work / wall time of the K = --steps back-to-back steps, bracketed by one
+             event pair on the launch stream, after max(--warmup, 10) untimed steps
+  timing     100 further iterations in 20 batches: median / p10 / p90 of the per-step time
+  roofline   the dominant kernel: algorithmic bytes (or FLOPs) per launch / its median launch
+             duration from events on the launch stream (for the single-kernel workloads a step
+             IS that launch; the MoE GEMMs and the two gating kernels are timed in passes of
+             their own); `traffic` (HBM bytes per launch from rocprofv3 --pmc, a separate run)
+             is read from profiles/hbm_traffic.json when a measurement has been committed
   cpu_baseline  the CPU oracle (a port of the reference's PyTorch ground truth) timed on a
-             bounded sample of the same workload on this host's cores
+             bounded sample of the same workload on this host's cores (model string included)
 """
 from __future__ import annotations
 
@@ -65,13 +68,30 @@ class Timer:
         return sum(a.elapsed_time(b) for a, b in self.pairs) / max(len(self.pairs), 1)
 
 
+MIN_WARMUP = 10       # warm-up iterations before any timed region, whatever --warmup says
+STAT_ITERS = 100      # iterations behind the median / p10 / p90 figures
+STAT_BATCHES = 20
+
+
+def _percentile(sorted_vals, q):
+    if not sorted_vals:
+        return None
+    pos = q * (len(sorted_vals) - 1)
+    lo, hi = int(math.floor(pos)), int(math.ceil(pos))
+    return sorted_vals[lo] + (sorted_vals[hi] - sorted_vals[lo]) * (pos - lo)
+
+
 def _time_steps(step, steps, warmup):
-    """step(i) launches one step; returns (ms_per_step, ms_per_step): the K steps are bracketed
-    by one event before and one after on the launch stream, and nothing else is recorded inside
-    the region (an event pair around every step costs about 10 us of host time and 7 us of GPU
-    time per step -- a quarter of the shortest workload).  For a single-kernel workload the
-    region divided by K is also that kernel's average launch duration, launch gaps included."""
-    for i in range(warmup):
+    """step(i) launches one step.  Returns (ms_per_step, stats).
+
+    ms_per_step: the K = `steps` timed steps are bracketed by one event before and one after on
+    the launch stream, and nothing else is recorded inside the region (an event pair around every
+    step costs about 10 us of host time and 7 us of GPU time per step -- a quarter of the shortest
+    workload).  At least MIN_WARMUP untimed steps run first.
+    stats: STAT_ITERS further iterations in STAT_BATCHES batches, one event pair per batch; the
+    median / p10 / p90 are over the per-step times of the batches (batch time / batch size).  For
+    a single-kernel workload a step is that kernel's launch, launch gaps included."""
+    for i in range(max(warmup, MIN_WARMUP)):
         step(i)
     torch.cuda.synchronize()
     t_all = Timer()
@@ -81,10 +101,46 @@ def _time_steps(step, steps, warmup):
     t_all.stop(ev)
     torch.cuda.synchronize()
     ms = t_all.mean_ms() / steps
-    return ms, ms
+    return ms, _batch_stats(step)
+
+
+def _batch_stats(step, iters=STAT_ITERS, batches=STAT_BATCHES):
+    per = max(1, -(-iters // batches))
+    tb = Timer()
+    n = 0
+    for _ in range(batches):
+        ev = tb.start()
+        for _ in range(per):
+            step(n)
+            n += 1
+        tb.stop(ev)
+    torch.cuda.synchronize()
+    vals = sorted(a.elapsed_time(b) / per for a, b in tb.pairs)
+    return {"iterations": n, "batch": per, "median_ms": _percentile(vals, 0.5),
+            "p10_ms": _percentile(vals, 0.1), "p90_ms": _percentile(vals, 0.9)}
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _cpu_info(cores=None):
+    return {"cores": cores if cores is not None else torch.get_num_threads(),
+            "cpu_model": _cpu_model(), "cpu_count": os.cpu_count()}
 
 
 def _traffic(name):
+    """HBM bytes per launch of the named kernel from the committed rocprofv3 --pmc summary (a
+    separate run: counters cannot be read inside this process), or None."""
+    if name is None:
+        return None
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
@@ -106,10 +162,11 @@ def wl_silu(dev, steps, warmup, cpu):
     outs = [torch.empty((M, N), dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
     bytes_ = M * 2 * N * 2 + M * N * 2
 
-    ms, ms_kernel = _time_steps(lambda i: silu_and_mul(xs[i % nbuf], outs[i % nbuf]), steps, warmup)
+    ms, st = _time_steps(lambda i: silu_and_mul(xs[i % nbuf], outs[i % nbuf]), steps, warmup)
+    ms_kernel = st["median_ms"]
     res = {
         "metric": "silu_and_mul HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
-        "ms_per_step": ms, "dtype": "bf16",
+        "ms_per_step": ms, "timing": st, "dtype": "bf16",
         "config": {"workload": "silu_and_mul bf16 [8192, 2x11008] N(0,1) seed 0"},
         "roofline": {"kernel": "silu_and_mul_vec16", "bound": "hbm",
                      "achieved": bytes_ / ms_kernel / 1e6, "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -128,7 +185,7 @@ def wl_silu(dev, steps, warmup, cpu):
             oa.silu_and_mul(sample)
         dt = (time.perf_counter() - t0) / reps
         res["cpu_baseline"] = {"value": bytes_ * rows / M / dt / 1e9, "unit": "GB/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"{rows} of {M} rows, {reps} reps"}
     return res
 
@@ -179,33 +236,32 @@ def wl_gating(dev, steps, warmup, cpu):
     npad = step(0)[4]
     l_pad = int(npad.item())
     bytes_ = (T * E * 4 + T * K * 4 * 2 + T * K * 4 + 4 * l_pad + 4 * l_pad // BLK + E * 4 + 4)
-    ms, _ = _time_steps(step, steps, warmup)
+    ms, st = _time_steps(step, steps, warmup)
     ms_two, _ = _time_steps(step_two_calls, steps, warmup)
 
-    # the same call replayed from a HIP graph (no Python / launch latency in between)
-    graph_ms = _graph_replay_ms(lambda: step(0), steps, warmup, "gating")
-
-    # dominant kernel: the router (reads the logits, 72% of the bytes)
-    tk = Timer()
-    for i in range(steps):
-        e = tk.start()
-        moe_topk_softmax(logits, K)
-        tk.stop(e)
-    ms_router = tk.mean_ms()
-    router_bytes = T * E * 4 + T * K * 8
+    # GPU time of the call itself (its two kernels and the gap between them), without the host
+    # between calls: N calls captured into one HIP graph, replayed; a graph of ONE call replayed
+    # shows what a graph launch itself costs on this stack
+    calls = 20
+    graph_ms = _graph_replay_ms(lambda: [step(0) for _ in range(calls)][-1], 20, 5, "gating")
+    graph1_ms = _graph_replay_ms(lambda: step(0), 20, 5, "gating (one call per graph)")
+    ms_gpu = graph_ms / calls if graph_ms is not None else st["median_ms"]
     res = {
         "metric": "MoE gating HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
-        "ms_per_step": ms, "dtype": "f32",
+        "ms_per_step": ms, "timing": st, "dtype": "f32",
         "config": {"workload": "moe_topk_softmax_align (router + alignment) fp32 [16384, 64] k=6 block 64 seed 1",
                    "padded_len": l_pad, "algorithmic_bytes": bytes_},
         "two_separate_calls": {"ms_per_step": ms_two, "value": bytes_ / ms_two / 1e6, "unit": "GB/s"},
         "graph_replay": None if graph_ms is None else {
-            "ms_per_step": graph_ms, "value": bytes_ / graph_ms / 1e6, "unit": "GB/s"},
-        "roofline": {"kernel": "moe_topk_softmax_kernel", "bound": "hbm",
-                     "achieved": router_bytes / ms_router / 1e6, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": router_bytes / ms_router / 1e6 / PEAK_HBM_GBS,
-                     "traffic": _traffic("moe_topk_softmax"),
-                     "note": "4 MB working set: launch-latency bound, served from cache"},
+            "calls_per_graph": calls, "ms_per_call": ms_gpu, "value": bytes_ / ms_gpu / 1e6,
+            "unit": "GB/s",
+            "one_call_per_graph_ms": graph1_ms},
+        "roofline": {"kernel": "moe_topk_softmax_count_kernel + align_place_fused_kernel (the two "
+                               "kernels of one call; GPU time per call from a graph of 20 calls)",
+                     "bound": "hbm", "achieved": bytes_ / ms_gpu / 1e6, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": bytes_ / ms_gpu / 1e6 / PEAK_HBM_GBS,
+                     "traffic": _traffic("moe_gating"),
+                     "note": "5.8 MB working set: launch-latency bound, served from cache"},
     }
     if cpu:
         from oracle import moe_gating as og
@@ -217,7 +273,7 @@ def wl_gating(dev, steps, warmup, cpu):
             og.align_block_size(ids, BLK, E)
         dt = (time.perf_counter() - t0) / reps
         res["cpu_baseline"] = {"value": bytes_ / dt / 1e9, "unit": "GB/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"full workload, {reps} reps"}
     return res
 
@@ -239,11 +295,12 @@ def wl_prefill(dev, steps, warmup, cpu):
     max_len = int(lens.max())
     flops = 4 * 128 * 32 * sum(int(l) * (int(l) + 1) // 2 for l in lens)
 
-    ms, ms_kernel = _time_steps(
+    ms, st = _time_steps(
         lambda i: context_attention_fwd(q, k, v, o, start, seqlen, max_len), steps, warmup)
+    ms_kernel = st["median_ms"]
     res = {
         "metric": "prefill attention TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
-        "ms_per_step": ms, "dtype": "bf16",
+        "ms_per_step": ms, "timing": st, "dtype": "bf16",
         "config": {"workload": "context_attention_fwd causal varlen, 8 seqs U[512,4096] seed 2, "
                                "32q/8kv heads, d128, bf16", "total_tokens": total,
                    "algorithmic_flops": flops},
@@ -262,7 +319,7 @@ def wl_prefill(dev, steps, warmup, cpu):
         dt = time.perf_counter() - t0
         sflops = 4 * 128 * 32 * L * (L + 1) // 2
         res["cpu_baseline"] = {"value": sflops / dt / 1e12, "unit": "TFLOP/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"one {L}-token sequence, 32 heads, 1 rep"}
     return res
 
@@ -297,10 +354,11 @@ def wl_decode(dev, steps, warmup, cpu):
     def step(i):
         paged_attention_fwd(q, kcs[i % nbuf], vcs[i % nbuf], o, table_d, None, ones, ctx_d, 1)
 
-    ms, ms_kernel = _time_steps(step, steps, warmup)
+    ms, st = _time_steps(step, steps, warmup)
+    ms_kernel = st["median_ms"]
     res = {
         "metric": "paged decode attention HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
-        "ms_per_step": ms, "dtype": "bf16", "tflops": flops / ms / 1e9,
+        "ms_per_step": ms, "timing": st, "dtype": "bf16", "tflops": flops / ms / 1e9,
         "config": {"workload": "paged_attention_fwd decode, batch 64, ctx U[512,8192] seed 3, "
                                "64-token pages, 32q/8kv heads, d128, bf16",
                    "sum_ctx": sum_ctx, "algorithmic_bytes": bytes_},
@@ -318,13 +376,15 @@ def wl_decode(dev, steps, warmup, cpu):
         dt = time.perf_counter() - t0
         sbytes = int(ctx[:n].sum()) * HKV * D * 4
         res["cpu_baseline"] = {"value": sbytes / dt / 1e9, "unit": "GB/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"first {n} of {B} sequences, 1 rep"}
     return res
 
 
 def wl_moe_fp8(dev, steps, warmup, cpu):
-    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8, shuffle_moe_weight_fp8
+    from dlcompiler_amd import _lib
+    from dlcompiler_amd.kernels import fused_moe as fm
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size
     from oracle import fp8 as ofp8
     from oracle import moe_gating as og
 
@@ -341,47 +401,71 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         w1q[e], w1s[e] = ofp8.block_quant_weight(torch.randn((2 * I, H), generator=g) * 0.02)
         w2q[e], w2s[e] = ofp8.block_quant_weight(torch.randn((H, I), generator=g) * 0.02)
     x, tw, ids = x_cpu.to(dev), tw_cpu.to(dev), ids_cpu.to(dev)
-    dw = [t.to(dev) for t in (w1q, w1s, w2q, w2s)]
-    # weights are re-arranged once at load time into MFMA-operand order (untimed, like the
-    # offline quantisation); DLB_BENCH_PLAIN_WEIGHTS=1 times the row-major layout instead
-    shuffled = os.environ.get("DLB_BENCH_PLAIN_WEIGHTS", "0") != "1"
-    if shuffled:
-        dw[0], dw[2] = shuffle_moe_weight_fp8(dw[0]), shuffle_moe_weight_fp8(dw[2])
+    plain = [t.to(dev) for t in (w1q, w1s, w2q, w2s)]
+    # operand order: the weights re-arranged once at load time (untimed, like the quantisation)
+    shuf = [fm.shuffle_moe_weight_fp8(plain[0]), plain[1], fm.shuffle_moe_weight_fp8(plain[2]), plain[3]]
     flops = 2 * T * K * H * 2 * I + 2 * T * K * I * H
-    gate_up_flops = 2 * T * K * H * 2 * I
+    gate_up_flops, down_flops = 2 * T * K * H * 2 * I, 2 * T * K * I * H
 
-    ms, _ = _time_steps(lambda i: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled),
-                        steps, warmup)
+    def kernel_times(dw, shuffled):
+        """Median duration of the two grouped-GEMM launches, each timed alone on the inputs the
+        step gives it (events around batches of launches of that one kernel)."""
+        lib = _lib.load()
+        block = fm._BLOCK_M
+        sorted_ids, _, _, counts = moe_align_block_size(ids, block, E, return_counts=True)
+        nmb = -(-sorted_ids.numel() // block)
+        xq, xs = fm.per_token_group_quant_fp8(x)
+        hq = torch.empty((nmb * block, I), dtype=torch.float8_e4m3fn, device=dev)
+        hs = torch.empty((nmb * block, I // 128), dtype=torch.float32, device=dev)
+        slots = torch.empty((T * K, H), dtype=torch.bfloat16, device=dev)
+        stream = _lib.current_stream_ptr(dev)
 
-    graph_ms = _graph_replay_ms(
-        lambda: fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled), steps, warmup, "moe")
+        def gate_up(i):
+            _lib.check(lib.dlb_moe_gemm_fp8_gate_up(
+                xq.data_ptr(), xs.data_ptr(), dw[0].data_ptr(), dw[1].data_ptr(), sorted_ids.data_ptr(),
+                counts.data_ptr(), E, nmb, block, T, K, H, I, 0, E, int(shuffled), hq.data_ptr(),
+                hs.data_ptr(), stream), "gate_up")
 
-    stage_t = {}
-    state = {"name": None, "ev": None}
+        def down(i):
+            _lib.check(lib.dlb_moe_gemm_fp8_down(
+                hq.data_ptr(), hs.data_ptr(), dw[2].data_ptr(), dw[3].data_ptr(), sorted_ids.data_ptr(),
+                counts.data_ptr(), E, tw.data_ptr(), nmb, block, T, K, H, I, 0, E, int(shuffled),
+                slots.data_ptr(), 0, stream), "down")
 
-    def hook(name):
-        if state["name"] is not None:
-            stage_t.setdefault(state["name"], Timer()).stop(state["ev"])
-        state["name"] = name
-        if name is not None:
-            state["ev"] = stage_t.setdefault(name, Timer()).start()
+        for i in range(MIN_WARMUP):
+            gate_up(i)
+            down(i)
+        return _batch_stats(gate_up), _batch_stats(down)
 
-    for i in range(steps):
-        fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled, _stage_hook=hook)
-    stages = {k: v.mean_ms() for k, v in stage_t.items()}
-    ms_gate_up = stages["gate_up"]
+    layouts = {}
+    for name, dw, shuffled in (("operand-order", shuf, True), ("row-major", plain, False)):
+        ms, st = _time_steps(lambda i: fm.fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled),
+                             steps, warmup)
+        graph_ms = _graph_replay_ms(
+            lambda: fm.fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled), 20, 5, "moe " + name)
+        st_gu, st_dn = kernel_times(dw, shuffled)
+        layouts[name] = {
+            "ms_per_step": ms, "value": flops / ms / 1e9, "unit": "TFLOP/s", "timing": st,
+            "graph_replay_ms": graph_ms,
+            "gate_up_kernel": dict(st_gu, tflops=gate_up_flops / st_gu["median_ms"] / 1e9,
+                                   frac=gate_up_flops / st_gu["median_ms"] / 1e9 / PEAK_FP8_TFLOPS),
+            "down_kernel": dict(st_dn, tflops=down_flops / st_dn["median_ms"] / 1e9,
+                                frac=down_flops / st_dn["median_ms"] / 1e9 / PEAK_FP8_TFLOPS),
+        }
+    best = layouts["operand-order"]
+    ms = best["ms_per_step"]
+    ms_gate_up = best["gate_up_kernel"]["median_ms"]
     res = {
         "metric": "fp8 fused-MoE TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
-        "ms_per_step": ms, "dtype": "fp8_e4m3",
+        "ms_per_step": ms, "timing": best["timing"], "dtype": "fp8_e4m3",
         "config": {"workload": "fused_moe_fp8 T=4096 H=2048 I=1408 E=64 top-6, fp8 e4m3 weights "
                                "128x128 block scales, per-token-group act quant, seed 5",
-                   "weight_layout": "operand-order" if shuffled else "row-major",
+                   "weight_layout": "operand-order (re-arranged once at load time; the reference's "
+                                    "row-major layout is under weight_layouts)",
                    "algorithmic_flops": flops},
-        "stages_ms": stages,
-        "graph_replay": None if graph_ms is None else {
-            "ms_per_step": graph_ms, "value": flops / graph_ms / 1e9, "unit": "TFLOP/s"},
-        "gemm_only_tflops": flops / (stages["gate_up"] + stages["down"]) / 1e9,
-        "roofline": {"kernel": "moe_gemm_fp8_kernel<gate_up>", "bound": "mfma",
+        "weight_layouts": layouts,
+        "gemm_only_tflops": flops / (ms_gate_up + best["down_kernel"]["median_ms"]) / 1e9,
+        "roofline": {"kernel": "moe_gemm_kernel<gate_up>", "bound": "mfma",
                      "achieved": gate_up_flops / ms_gate_up / 1e9, "peak": PEAK_FP8_TFLOPS,
                      "unit": "TFLOP/s", "frac": gate_up_flops / ms_gate_up / 1e9 / PEAK_FP8_TFLOPS,
                      "traffic": _traffic("moe_gemm_fp8_gate_up")},
@@ -398,18 +482,20 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
             reps += 1
         dt = (time.perf_counter() - t0) / reps
         res["cpu_baseline"] = {"value": flops / dt / 1e12, "unit": "TFLOP/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"all {T} tokens, {reps} reps ({dt * reps:.1f} s of CPU time)"}
     return res
 
 
-def _hbm_result(metric, workload, bytes_, ms, ms_kernel, kernel, dtype="bf16"):
+def _hbm_result(metric, workload, bytes_, ms, st, kernel, dtype="bf16", traffic=None):
+    ms_kernel = st["median_ms"]
     return {
         "metric": metric, "unit": "GB/s", "value": bytes_ / ms / 1e6, "ms_per_step": ms,
+        "timing": st,
         "dtype": dtype, "config": {"workload": workload, "algorithmic_bytes": bytes_},
         "roofline": {"kernel": kernel, "bound": "hbm", "achieved": bytes_ / ms_kernel / 1e6,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": bytes_ / ms_kernel / 1e6 / PEAK_HBM_GBS, "traffic": None},
+                     "frac": bytes_ / ms_kernel / 1e6 / PEAK_HBM_GBS, "traffic": _traffic(traffic)},
     }
 
 
@@ -430,7 +516,7 @@ def wl_add_rms_norm(dev, steps, warmup, cpu):
                                              out=outs[i % nbuf], out_residual=ors[i % nbuf]),
                           steps, warmup)
     res = _hbm_result("add_rms_norm HBM GB/s", "rms_norm with residual, bf16 [16384, 4096] seed 6",
-                      bytes_, ms, msk, "rms_norm_kernel<add>")
+                      bytes_, ms, msk, "rms_norm_kernel<add>", traffic="add_rms_norm")
     if cpu:
         from oracle import decoder_ops as od
 
@@ -439,7 +525,7 @@ def wl_add_rms_norm(dev, steps, warmup, cpu):
         od.rms_norm(x, w.cpu(), 1e-6, residual=r)
         dt = time.perf_counter() - t0
         res["cpu_baseline"] = {"value": bytes_ * 2048 / M / dt / 1e9, "unit": "GB/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"2048 of {M} rows, 1 rep"}
     return res
 
@@ -462,7 +548,7 @@ def wl_rotary(dev, steps, warmup, cpu):
                                                          qo[i % nbuf], ko[i % nbuf]), steps, warmup)
     res = _hbm_result("apply_rotary_pos_emb HBM GB/s",
                       "apply_rotary_pos_emb bf16 q [16384, 32, 128], k [16384, 8, 128] seed 7",
-                      bytes_, ms, msk, "rotary_kernel")
+                      bytes_, ms, msk, "rotary_kernel", traffic="apply_rotary_pos_emb")
     if cpu:
         from oracle import decoder_ops as od
 
@@ -471,7 +557,7 @@ def wl_rotary(dev, steps, warmup, cpu):
         od.apply_rotary_pos_emb(qs[0][:n].cpu(), ks[0][:n].cpu(), cos[:n, None].cpu(), sin[:n, None].cpu())
         dt = time.perf_counter() - t0
         res["cpu_baseline"] = {"value": bytes_ * n / T / dt / 1e9, "unit": "GB/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": f"{n} of {T} tokens, 1 rep"}
     return res
 
@@ -506,7 +592,7 @@ def wl_fill_kv_cache(dev, steps, warmup, cpu):
                           steps, warmup)
     res = _hbm_result("fill_kv_cache HBM GB/s",
                       f"fill_kv_cache bf16, 8 seqs U[512,4096] seed 2 ({T} tokens), 8 kv heads, d128, 64-token pages",
-                      bytes_, ms, msk, "fill_kv_cache_kernel")
+                      bytes_, ms, msk, "fill_kv_cache_kernel", traffic="fill_kv_cache")
     if cpu:
         from oracle import decoder_ops as od
 
@@ -515,7 +601,7 @@ def wl_fill_kv_cache(dev, steps, warmup, cpu):
                          [int(lens[0])], [0], table[:1])
         dt = time.perf_counter() - t0
         res["cpu_baseline"] = {"value": bytes_ * int(lens[0]) / T / dt / 1e9, "unit": "GB/s",
-                               "cores": 1, "kind": "port",
+                               **_cpu_info(1), "kind": "port",
                                "sample": f"first sequence ({int(lens[0])} tokens), 1 rep (includes a copy of the cache)"}
     return res
 
@@ -546,17 +632,19 @@ def wl_paged_prefill(dev, steps, warmup, cpu):
     kvl_d, table_d = kvl.to(torch.int32).to(dev), table.to(dev)
     pairs = sum(QL * int(h) + QL * (QL + 1) // 2 for h in hist)
     flops = 4 * D * HQ * pairs
-    ms, msk = _time_steps(lambda i: paged_attention_fwd(q, kc, vc, o, table_d, start, ql, kvl_d, QL),
-                          steps, warmup)
+    ms, st = _time_steps(lambda i: paged_attention_fwd(q, kc, vc, o, table_d, start, ql, kvl_d, QL),
+                         steps, warmup)
+    msk = st["median_ms"]
     res = {
         "metric": "paged prefill attention TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
-        "ms_per_step": ms, "dtype": "bf16",
+        "ms_per_step": ms, "timing": st, "dtype": "bf16",
         "config": {"workload": "paged_attention_fwd prefill, 8 seqs x 512 new tokens after history "
                                "U[512,4096] seed 8, 64-token pages, 32q/8kv heads, d128, bf16",
                    "algorithmic_flops": flops},
         "roofline": {"kernel": "prefill_attn_kernel<paged>", "bound": "mfma",
                      "achieved": flops / msk / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / msk / 1e9 / PEAK_BF16_TFLOPS, "traffic": None},
+                     "frac": flops / msk / 1e9 / PEAK_BF16_TFLOPS,
+                     "traffic": _traffic("paged_prefill")},
     }
     if cpu:
         from oracle import attention as oa
@@ -567,7 +655,7 @@ def wl_paged_prefill(dev, steps, warmup, cpu):
         dt = time.perf_counter() - t0
         f1 = 4 * D * HQ * (QL * int(hist[0]) + QL * (QL + 1) // 2)
         res["cpu_baseline"] = {"value": f1 / dt / 1e12, "unit": "TFLOP/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               **_cpu_info(), "kind": "port",
                                "sample": "first sequence, 1 rep"}
     return res
 
@@ -590,8 +678,8 @@ PRIMARY = "moe_fp8"
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -637,7 +725,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": p["dtype"],
         "data": "synthetic", "config": p["config"], "roofline": p["roofline"],
         "cpu_baseline": p.get("cpu_baseline"),
-        "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
+        "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
+                 "cpu_model": _cpu_model()},
         "workloads": results,
     }
     print(json.dumps(line))

@@ -37,11 +37,11 @@ SIGNATURES = {
                                                c_int64, c_void_p, c_void_p, c_void_p, c_size_t,
                                                c_void_p]),
     "dlb_paged_decode_ws_bytes": (c_size_t, [c_int] * 6),
-    "dlb_paged_decode_attn": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_int64] * 11
+    "dlb_paged_decode_attn": (c_int, [c_void_p] * 6 + [c_int] * 7 + [c_int64] * 11
                               + [c_float, c_int, c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "dlb_prefill_attn_varlen": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 8
                                 + [c_float, c_int, c_void_p]),
-    "dlb_paged_prefill_attn": (c_int, [c_void_p] * 8 + [c_int] * 7 + [c_int64] * 11
+    "dlb_paged_prefill_attn": (c_int, [c_void_p] * 8 + [c_int] * 8 + [c_int64] * 11
                                + [c_float, c_int, c_float, c_int, c_void_p]),
     "dlb_per_token_group_quant_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                               c_int64, c_int64, c_int64, c_int, c_void_p]),

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/dlblas_hip.h"
 
 namespace dlb {
@@ -226,6 +228,23 @@ inline int route_chunk_tokens(int64_t T) { return (T + 63) / 64 <= kRouteMaxChun
 int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
                               int K, int64_t ld_logits, int renormalize, int chunk_tokens,
                               int32_t* chunk_counts, hipStream_t s);
+
+// compute units of the device that is current on this thread (256 if it cannot be read), kept
+// per device: a process may drive GPUs of different sizes.  The table is filled lazily; two
+// threads racing on one entry write the same value.
+inline int current_device_cu_count() {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> table[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = table[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    table[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
 
 // status of the launch just issued on this thread
 inline int launch_status() { return hipGetLastError() == hipSuccess ? DLB_OK : DLB_ERR_LAUNCH; }

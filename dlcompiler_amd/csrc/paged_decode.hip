@@ -48,6 +48,7 @@ struct DecodeParams {
   int num_teams;
   float scale_log2e;
   float sm_scale;
+  int dk, dv;      // real key / value head sizes (<= the padded size the kernel is built for)
   int window;      // > 0: keys older than (ctx - 1 - window) are masked (paged_attention.py:163-167)
   float softcap;   // > 0: logits -> softcap * tanh(logits / softcap) (paged_attention.py:186-189)
 };
@@ -84,8 +85,16 @@ struct Mma16<DLB_DTYPE_F16> {
 constexpr int kTile = 64;          // keys per iteration
 constexpr int kVtRowBytes = 144;   // 64 keys * 2 B + 16 B pad
 
-template <int DT, int D, bool POW2>
-__global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeParams p) {
+// D is the padded head size the kernel is built for (64 or 128).  RAGGED: the real key size dk
+// and / or value size dv is smaller (any multiple of 8): query dims past dk are zero, so whatever
+// the key loads of those dims return does not count -- they are redirected to the row's first 16
+// bytes to stay inside the cache -- and value dims past dv (redirected likewise) only produce
+// output dims that are never stored.  The reference splits odd head sizes the same way into
+// power-of-two blocks with masked loads (python/dlBLAS/dlblas/kernels/paged_attention.py:531-539).
+// (The masked variant keeps a few more per-lane offsets alive: it is built for one wavefront per
+// SIMD instead of two rather than spilling them.)
+template <int DT, int D, bool POW2, bool RAGGED>
+__global__ __launch_bounds__(64, RAGGED ? 1 : 2) void paged_decode_split_kernel(const DecodeParams p) {
   constexpr int KS = D / 32;   // MFMA k-steps over the head dim
   constexpr int MT = D / 16;   // 16-row tiles of O^T
   constexpr int DG = D / 8;    // 8-dim groups per key row
@@ -144,7 +153,7 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     qf[ks] = u32x4{0u, 0u, 0u, 0u};
-    if (head_ok)
+    if (head_ok && (!RAGGED || 32 * ks + 8 * g < p.dk))
       qf[ks] = *(const u32x4*)(qb + (int64_t)b * p.q_sb + (int64_t)head * p.q_sh + 32 * ks + 8 * g);
   }
 
@@ -163,6 +172,11 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
   constexpr int VL = 64 / DG < 4 ? 64 / DG : 4;  // 4-key groups of a sub-tile staged per pass
   constexpr int VPASS = 4 / VL;                  // passes per 16-key sub-tile
   const int dg = lane % DG, kgl = lane / DG;     // lanes with kgl >= VL idle (D < 128)
+  // byte offsets of this lane's 16-byte pieces inside a key / value row
+  uint32_t kdim_off[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) kdim_off[ks] = (!RAGGED || 32 * ks + 8 * g < p.dk) ? 64u * ks + 16u * g : 0u;
+  const uint32_t vdim_off = (!RAGGED || 8 * dg < p.dv) ? 16u * dg : 0u;
 
   // The chunk is walked in half tiles of 32 keys (one k-step of the second product).  The loads
   // of half tile h + 1 are issued before half tile h is computed, so every wave keeps 16 KB of
@@ -207,9 +221,12 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
         const unsigned char* base = kbytes + pg * p.k_sp * 2;
         // K rows are read as two half-line (64-byte) pieces by consecutive k-steps: keep them
         // cacheable so the second piece hits the line the first one brought in
-        const uint32_t off = (uint32_t)(key - page_key0) * k_tok_bytes + 16u * g;
+        const uint32_t off = (uint32_t)(key - page_key0) * k_tok_bytes;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) f.kf[sub][ks] = *(const u32x4*)(base + off + 64 * ks);
+        for (int ks = 0; ks < KS; ++ks) {
+          if (RAGGED) f.kf[sub][ks] = *(const u32x4*)(base + off + kdim_off[ks]);
+          else f.kf[sub][ks] = *(const u32x4*)(base + off + 16u * g + 64 * ks);
+        }
       }
       {
         const unsigned char* base = vbytes + pg * p.v_sp * 2;
@@ -220,7 +237,7 @@ __global__ __launch_bounds__(64, 2) void paged_decode_split_kernel(const DecodeP
           if (kgl < VL) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const uint32_t off = (uint32_t)(key0 - page_key0 + min(r, room)) * v_tok_bytes + 16u * dg;
+              const uint32_t off = (uint32_t)(key0 - page_key0 + min(r, room)) * v_tok_bytes + vdim_off;
               f.vr[sub][ps][r] = __builtin_nontemporal_load((const u32x4*)(base + off));
             }
           }
@@ -437,7 +454,7 @@ __global__ __launch_bounds__(D) void paged_decode_combine_kernel(const DecodePar
     }
     acc /= den;
   }
-  Elem<DT>::store1(p.o, (int64_t)b * p.o_sb + (int64_t)head * p.o_sh + d, acc);
+  if (d < p.dv) Elem<DT>::store1(p.o, (int64_t)b * p.o_sb + (int64_t)head * p.o_sh + d, acc);
 }
 
 // smallest piece a team may get, in 32-key units: 512 keys, less for small problems so that
@@ -458,16 +475,7 @@ int partial_slots(int max_ctx, int min_units) {
 
 // teams that are resident together: 8 wavefronts per CU (2 per SIMD) / wavefronts per team
 int pick_num_teams(int units_per_team) {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cus = n;
-    else
-      cus = 256;
-  }
-  return max(1, cus * 8 / units_per_team);
+  return max(1, current_device_cu_count() * 8 / units_per_team);
 }
 
 }  // namespace
@@ -475,7 +483,8 @@ int pick_num_teams(int units_per_team) {
 
 extern "C" size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int page,
                                             int max_blocks) {
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || page <= 0 || max_blocks <= 0) return 0;
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || D > 128 || page <= 0 || max_blocks <= 0) return 0;
+  D = D <= 64 ? 64 : 128;  // the head size the kernels are built for
   const int group = Hq / Hkv;
   const int hchunks = (group + 15) / 16;
   const int64_t max_ctx = (int64_t)page * max_blocks;
@@ -486,8 +495,8 @@ extern "C" size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int p
 
 extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache,
                                      void* o, const int32_t* block_table, const int32_t* kv_len,
-                                     int B, int Hq, int Hkv, int D, int page, int max_blocks,
-                                     int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page,
+                                     int B, int Hq, int Hkv, int D, int Dv, int page,
+                                     int max_blocks, int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page,
                                      int64_t k_stride_tok, int64_t k_stride_head,
                                      int64_t v_stride_page, int64_t v_stride_tok,
                                      int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
@@ -495,11 +504,13 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
                                      float logit_softcapping, int dtype, void* ws,
                                      size_t ws_bytes, void* stream) {
   using namespace dlb;
-  if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || page < 1 || max_blocks < 1) return DLB_ERR_BAD_ARG;
+  if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || Dv < 1 || page < 1 || max_blocks < 1) return DLB_ERR_BAD_ARG;
   if (Hq % Hkv != 0) return DLB_ERR_BAD_ARG;
   if (B == 0) return DLB_OK;
   if (!q || !k_cache || !v_cache || !o || !block_table || !kv_len) return DLB_ERR_BAD_ARG;
-  if (D != 64 && D != 128) return DLB_ERR_UNSUPPORTED;
+  if (D % 8 != 0 || Dv % 8 != 0 || D > 128 || Dv > 128) return DLB_ERR_UNSUPPORTED;
+  const int Dp = (D <= 64 && Dv <= 64) ? 64 : 128;  // head size the kernel instance is built for
+  const bool ragged = D != Dp || Dv != Dp;
   if (page % 16 != 0) return DLB_ERR_UNSUPPORTED;
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
   if ((int64_t)page * max_blocks > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
@@ -512,7 +523,7 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
                              k_stride_head, v_stride_page, v_stride_tok,  v_stride_head};
   for (int64_t sd : strides)
     if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
-  const size_t need = dlb_paged_decode_ws_bytes(B, Hq, Hkv, D, page, max_blocks);
+  const size_t need = dlb_paged_decode_ws_bytes(B, Hq, Hkv, Dp, page, max_blocks);
   if (!ws || ws_bytes < need) return DLB_ERR_WORKSPACE;
 
   DecodeParams p;
@@ -550,8 +561,10 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   p.sm_scale = sm_scale;
   p.window = window_size;
   p.softcap = logit_softcapping;
+  p.dk = D;
+  p.dv = Dv;
   p.ws_o = (float*)ws;
-  p.ws_ml = p.ws_o + (size_t)B * Hq * p.nsplit_max * D;
+  p.ws_ml = p.ws_o + (size_t)B * Hq * p.nsplit_max * Dp;
   p.ws_np = (int32_t*)(p.ws_ml + (size_t)B * Hq * p.nsplit_max * 2);
 
   hipStream_t s = (hipStream_t)stream;
@@ -560,23 +573,27 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   if (units > 65535 || p.num_teams > 65535) return DLB_ERR_UNSUPPORTED;
   const dim3 grid1((uint32_t)units, (uint32_t)p.num_teams);
   const dim3 grid2((uint32_t)Hq, (uint32_t)B);
-#define DLB_LAUNCH_DECODE(DT_, D_)                                                          \
-  do {                                                                                      \
-    if (p.page_shift >= 0)                                                                  \
-      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, true>), grid1, dim3(64), 0, \
-                         s, p);                                                             \
-    else                                                                                    \
-      hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, false>), grid1, dim3(64),   \
-                         0, s, p);                                                          \
-    hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p);   \
+#define DLB_LAUNCH_SPLIT(DT_, D_, P2_, RG_) \
+  hipLaunchKernelGGL((paged_decode_split_kernel<DT_, D_, P2_, RG_>), grid1, dim3(64), 0, s, p)
+#define DLB_LAUNCH_DECODE(DT_, D_)                                                        \
+  do {                                                                                    \
+    if (p.page_shift >= 0) {                                                              \
+      if (ragged) DLB_LAUNCH_SPLIT(DT_, D_, true, true);                                  \
+      else DLB_LAUNCH_SPLIT(DT_, D_, true, false);                                        \
+    } else {                                                                              \
+      if (ragged) DLB_LAUNCH_SPLIT(DT_, D_, false, true);                                 \
+      else DLB_LAUNCH_SPLIT(DT_, D_, false, false);                                       \
+    }                                                                                     \
+    hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p); \
   } while (0)
   if (dtype == DLB_DTYPE_BF16) {
-    if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 128);
+    if (Dp == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 128);
     else DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 64);
   } else {
-    if (D == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
+    if (Dp == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
     else DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 64);
   }
+#undef DLB_LAUNCH_SPLIT
 #undef DLB_LAUNCH_DECODE
   return launch_status();
 }

@@ -43,6 +43,7 @@ struct PrefillParams {
   const int32_t* block_table;
   int64_t bt_stride, k_sp, v_sp;
   int page, page_shift;
+  int dk, dv;  // real key / value head sizes (<= the padded size D the kernel is built for)
   // generic masking (both layouts): sliding window (> 0) and logit soft-cap (> 0)
   int window;
   float softcap, sm_scale;
@@ -89,11 +90,15 @@ struct Smem {
   static constexpr int stage = kBytes + vBytes;
 };
 
-#ifndef DLB_PF_OCC
-#define DLB_PF_OCC 2
-#endif
-template <int DT, int D, bool PAGED>
-__global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(const PrefillParams p) {
+// D is the padded head size the kernel is built for (64 or 128).  RAGGED: the real key size dk
+// and / or value size dv is smaller (any multiple of 8): the query dims past dk are loaded as
+// zeros, so the key bytes staged for those dims do not count -- their copies are redirected to
+// the row's first 16 bytes to stay inside the tensor -- and value dims past dv (redirected
+// likewise) only produce output dims that are never stored.  The reference handles odd head
+// sizes by splitting them into power-of-two blocks with masked loads
+// (python/dlBLAS/dlblas/kernels/paged_attention.py:531-539).
+template <int DT, int D, bool PAGED, bool RAGGED>
+__global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int KS = D / 16;  // MFMA k-steps over the head dim for S^T
   constexpr int MT = D / 32;  // 32-row tiles of O^T
   constexpr int DG = D / 8;
@@ -105,7 +110,11 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
   // between the sequences of a batch while the grid holds only a few workgroups per slot, so
   // the sequences are walked longest context first (blockIdx.z = rank, not index): the long
   // ones start in the first round and the short ones fill in behind them.
-  int seq = blockIdx.z;
+  // Packed layout: a tile's cost is set by its position in its sequence alone, so the grid runs
+  // over (head, sequence, query tile) with the tile index slowest and reversed: the last tiles
+  // of the long sequences start first, everywhere, and the cheap first tiles of all sequences
+  // finish the launch.
+  int seq = PAGED ? blockIdx.z : blockIdx.y;
   if (PAGED && gridDim.z > 1 && gridDim.z <= kThreads) {
     __shared__ int32_t rank_key[kThreads];
     __shared__ int32_t rank_seq;
@@ -126,7 +135,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     seq = __builtin_amdgcn_readfirstlane(rank_seq);
   }
   const int L = p.seq_len[seq];
-  const int qtile = gridDim.y - 1 - blockIdx.y;  // heaviest tiles first
+  const int qtile = PAGED ? gridDim.y - 1 - blockIdx.y : gridDim.z - 1 - blockIdx.z;  // heaviest first
   const int q0 = qtile * kBlockM;
   if (q0 >= L) return;
   const int64_t tok0 = p.start_loc[seq];
@@ -155,7 +164,10 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     const unsigned short* qp =
         qb + (tok0 + min(qrow, L - 1)) * p.q_st + (int64_t)head * p.q_sh + 8 * hh;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qp + 16 * ks);
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = u32x4{0u, 0u, 0u, 0u};
+      if (!RAGGED || 16 * ks + 8 * hh < p.dk) qf[ks] = *(const u32x4*)(qp + 16 * ks);
+    }
   }
 
   const int kv_end = min(kv_total, hist + q0 + kBlockM);  // keys this workgroup needs
@@ -196,6 +208,16 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
     return D == 128 ? (((r & 3) << 2) | (((r >> 2) & 1) << 1))
                     : ((((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1));
   };
+  // byte offset inside its source row of the 16-byte chunk this lane copies into position k_pos
+  // of row r (the swizzle undone; chunks past the real head size fetch the row's first chunk)
+  auto k_chunk = [&](int r) -> unsigned int {
+    const int c = k_pos ^ (r & (DG - 1));
+    return (unsigned int)((RAGGED && 8 * c >= p.dk) ? 0 : c) << 4;
+  };
+  auto v_chunk = [&](int r) -> unsigned int {
+    const int c = k_pos ^ v_swz(r);
+    return (unsigned int)((RAGGED && 8 * c >= p.dv) ? 0 : c) << 4;
+  };
   // paged layout: the page ids of the rows this lane copies are fetched one tile ahead of the
   // copy that needs them, so the block-table latency never sits in front of a tile's copies
   int pg_next[KINS];
@@ -221,8 +243,8 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
 #pragma unroll
   for (int i = 0; i < KINS; ++i) {
     const int r = (4 * i + wave) * KRPI + k_lrow;
-    koff0[i] = (unsigned int)(r * k_row_bytes) + ((k_pos ^ (r & (DG - 1))) << 4);
-    voff0[i] = (unsigned int)(r * v_row_bytes) + ((k_pos ^ v_swz(r)) << 4);
+    koff0[i] = (unsigned int)(r * k_row_bytes) + k_chunk(r);
+    voff0[i] = (unsigned int)(r * v_row_bytes) + v_chunk(r);
   }
   unsigned int stage_dst = 0;
   auto prepare_tile = [&](auto clamp_tag, int t0, int buf) {
@@ -240,14 +262,12 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
         if (CLAMP) key = min(key, kv_total - 1);
         const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
         const int64_t slot = key - pi * p.page;
-        ksrc[i] = kbytes + ((int64_t)pg_next[i] * p.k_sp + slot * p.k_st) * 2 +
-                  ((k_pos ^ (r & (DG - 1))) << 4);
-        vsrc[i] = vbytes + ((int64_t)pg_next[i] * p.v_sp + slot * p.v_st) * 2 +
-                  ((k_pos ^ v_swz(r)) << 4);
+        ksrc[i] = kbytes + ((int64_t)pg_next[i] * p.k_sp + slot * p.k_st) * 2 + k_chunk(r);
+        vsrc[i] = vbytes + ((int64_t)pg_next[i] * p.v_sp + slot * p.v_st) * 2 + v_chunk(r);
       } else if (CLAMP) {
         const int rc = min(r, kv_total - 1 - t0);  // >= 0: a staged tile starts inside the context
-        koff[i] = (unsigned int)(rc * k_row_bytes) + ((k_pos ^ (r & (DG - 1))) << 4);
-        voff[i] = (unsigned int)(rc * v_row_bytes) + ((k_pos ^ v_swz(r)) << 4);
+        koff[i] = (unsigned int)(rc * k_row_bytes) + k_chunk(r);
+        voff[i] = (unsigned int)(rc * v_row_bytes) + v_chunk(r);
       } else {
         koff[i] = koff0[i];
         voff[i] = voff0[i];
@@ -455,7 +475,7 @@ __global__ __launch_bounds__(kThreads, DLB_PF_OCC) void prefill_attn_kernel(cons
         u32x2 w;
         w[0] = Mma32<DT>::pack2(o[mt][4 * qd + 0] * inv, o[mt][4 * qd + 1] * inv);
         w[1] = Mma32<DT>::pack2(o[mt][4 * qd + 2] * inv, o[mt][4 * qd + 3] * inv);
-        *(u32x2*)(op + 32 * mt + 8 * qd + 4 * hh) = w;
+        if (!RAGGED || 32 * mt + 8 * qd + 4 * hh < p.dv) *(u32x2*)(op + 32 * mt + 8 * qd + 4 * hh) = w;
       }
     }
   }
@@ -469,9 +489,13 @@ namespace {
 
 // Shared argument checks and launch of both entry points; the paged fields of `p` are already
 // filled in (or zeroed) by the caller.
-int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int D, int max_len,
+int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk, int Dv, int max_len,
                    float sm_scale, int dtype, void* stream) {
-  if (D != 64 && D != 128) return DLB_ERR_UNSUPPORTED;
+  if (Dk % 8 != 0 || Dv % 8 != 0 || Dk > 128 || Dv > 128) return DLB_ERR_UNSUPPORTED;
+  const int D = (Dk <= 64 && Dv <= 64) ? 64 : 128;  // head size the kernel instance is built for
+  const bool ragged = Dk != D || Dv != D;
+  p.dk = Dk;
+  p.dv = Dv;
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
   if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) ||
       (reinterpret_cast<uintptr_t>(p.o) & 7u) != 0)
@@ -494,10 +518,16 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int D, 
   p.sm_scale = sm_scale;
 
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((uint32_t)Hq, (uint32_t)ceil_div(max_len, kBlockM), (uint32_t)B);
-  if (grid.y > 65535) return DLB_ERR_UNSUPPORTED;
-#define DLB_LAUNCH_PREFILL(DT_, D_, PG_) \
-  hipLaunchKernelGGL((prefill_attn_kernel<DT_, D_, PG_>), grid, dim3(kThreads), 0, s, p)
+  const uint32_t qtiles = (uint32_t)ceil_div(max_len, kBlockM);
+  if (qtiles > 65535) return DLB_ERR_UNSUPPORTED;
+  const dim3 grid = paged ? dim3((uint32_t)Hq, qtiles, (uint32_t)B) : dim3((uint32_t)Hq, (uint32_t)B, qtiles);
+#define DLB_LAUNCH_PREFILL(DT_, D_, PG_)                                                          \
+  do {                                                                                            \
+    if (ragged)                                                                                   \
+      hipLaunchKernelGGL((prefill_attn_kernel<DT_, D_, PG_, true>), grid, dim3(kThreads), 0, s, p);  \
+    else                                                                                          \
+      hipLaunchKernelGGL((prefill_attn_kernel<DT_, D_, PG_, false>), grid, dim3(kThreads), 0, s, p); \
+  } while (0)
 #define DLB_DISPATCH_PREFILL(PG_)                              \
   if (dtype == DLB_DTYPE_BF16) {                               \
     if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 128, PG_); \
@@ -547,14 +577,14 @@ extern "C" int dlb_prefill_attn_varlen(const void* q, const void* k, const void*
   p.page_shift = 0;
   p.window = -1;
   p.softcap = -1.0f;
-  return launch_prefill(p, false, B, Hq, Hkv, D, max_len, sm_scale, dtype, stream);
+  return launch_prefill(p, false, B, Hq, Hkv, D, D, max_len, sm_scale, dtype, stream);
 }
 
 extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache,
                                       void* o, const int32_t* block_table,
                                       const int32_t* q_start_loc, const int32_t* q_len,
                                       const int32_t* kv_len, int B, int Hq, int Hkv, int D,
-                                      int page, int max_blocks, int max_q_len,
+                                      int Dv, int page, int max_blocks, int max_q_len,
                                       int64_t q_stride_tok, int64_t q_stride_head,
                                       int64_t k_stride_page, int64_t k_stride_tok,
                                       int64_t k_stride_head, int64_t v_stride_page,
@@ -563,7 +593,7 @@ extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const 
                                       int64_t bt_stride, float sm_scale, int window_size,
                                       float logit_softcapping, int dtype, void* stream) {
   using namespace dlb;
-  if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || max_q_len < 0 || page < 1 || max_blocks < 0)
+  if (B < 0 || Hq < 1 || Hkv < 1 || D < 1 || Dv < 1 || max_q_len < 0 || page < 1 || max_blocks < 0)
     return DLB_ERR_BAD_ARG;
   if (Hq % Hkv != 0) return DLB_ERR_BAD_ARG;
   if (B == 0 || max_q_len == 0) return DLB_OK;
@@ -593,5 +623,5 @@ extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const 
   p.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz((unsigned)page) : -1;
   p.window = window_size;
   p.softcap = logit_softcapping;
-  return launch_prefill(p, true, B, Hq, Hkv, D, max_q_len, sm_scale, dtype, stream);
+  return launch_prefill(p, true, B, Hq, Hkv, D, Dv, max_q_len, sm_scale, dtype, stream);
 }

@@ -29,7 +29,8 @@ def paged_attention_fwd(
     """Paged attention forward, written into ``o``; returns ``None`` like the reference.
 
     Args follow the reference: ``q`` [tokens, Hq, D]; ``k``/``v`` caches
-    [pages, page_size, Hkv, D]; ``block_offsets`` [batch, max_blocks] maps a sequence's
+    [pages, page_size, Hkv, D] / [pages, page_size, Hkv, Dv] (head sizes: multiples of 8 up to
+    128, the value size may differ from the key size; ``o`` is [tokens, Hq, Dv]); ``block_offsets`` [batch, max_blocks] maps a sequence's
     logical pages to physical ones; ``kv_seqlens`` [batch] context lengths.  One query token
     per sequence (``q.shape[-3] == q_seqlens.size(0)``, paged_attention.py:559) takes the
     split-KV decode kernel; anything else is the prefill-with-history case
@@ -42,13 +43,14 @@ def paged_attention_fwd(
     if logit_softcapping is None:
         logit_softcapping = -1.0
     Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
-    assert Lq == Lk, Lv == o.shape[-1]
+    assert Lq == Lk
+    assert Lv == o.shape[-1]
     if sm_scale is None:
         sm_scale = 1.0 / (Lq**0.5)
     batch, head = q_seqlens.shape[0], q.shape[-2]
     is_decoding = q.shape[-3] == q_seqlens.size(0)
-    if Lv != Lk:
-        raise NotImplementedError("value head size must equal key head size")
+    if Lk % 8 != 0 or Lv % 8 != 0 or Lk > 128 or Lv > 128:
+        raise NotImplementedError("head sizes must be multiples of 8, at most 128")
     assert k.dim() == 4 and v.dim() == 4 and k.shape[:3] == v.shape[:3]
     assert q.dtype == k.dtype == v.dtype == o.dtype
     num_kv_heads = k.shape[-2]
@@ -72,7 +74,7 @@ def paged_attention_fwd(
             st = lib.dlb_paged_prefill_attn(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), block_offsets.data_ptr(),
                 q_start_loc.data_ptr(), q_seqlens.data_ptr(), kv_seqlens.data_ptr(), batch, head,
-                num_kv_heads, Lq, page, max_blocks, int(max_seqlen), q.stride(0), q.stride(1),
+                num_kv_heads, Lq, Lv, page, max_blocks, int(max_seqlen), q.stride(0), q.stride(1),
                 k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
                 o.stride(0), o.stride(1), block_offsets.stride(0), float(sm_scale),
                 int(window_size), float(logit_softcapping), _lib.torch_dtype_code(q.dtype),
@@ -83,12 +85,12 @@ def paged_attention_fwd(
     q3 = q.reshape(batch, head, Lq) if q.dim() != 3 else q
     o3 = o.reshape(batch, head, Lv) if o.dim() != 3 else o
     assert o3.data_ptr() == o.data_ptr()
-    ws_bytes = lib.dlb_paged_decode_ws_bytes(batch, head, num_kv_heads, Lq, page, max_blocks)
+    ws_bytes = lib.dlb_paged_decode_ws_bytes(batch, head, num_kv_heads, max(Lq, Lv), page, max_blocks)
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=q.device)
     with _lib.device_guard(q.device):
         st = lib.dlb_paged_decode_attn(
             q3.data_ptr(), k.data_ptr(), v.data_ptr(), o3.data_ptr(), block_offsets.data_ptr(),
-            kv_seqlens.data_ptr(), batch, head, num_kv_heads, Lq, page, max_blocks,
+            kv_seqlens.data_ptr(), batch, head, num_kv_heads, Lq, Lv, page, max_blocks,
             q3.stride(0), q3.stride(1), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), o3.stride(0), o3.stride(1),
             block_offsets.stride(0), float(sm_scale), int(window_size), float(logit_softcapping),

@@ -129,8 +129,9 @@ int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t*
  * Replaces the decode branch of paged_attention_fwd, kernels/paged_attention.py:604-671
  * (_fwd_grouped_split_kernel :45-234 and _reduce_split_kernel :238-285).
  *   q            [B, Hq, D]            strides q_stride_b, q_stride_h, unit last stride
- *   k/v cache    [pages, page, Hkv, D] strides *_stride_page, *_stride_tok, *_stride_head
- *   o            [B, Hq, D]            strides o_stride_b, o_stride_h
+ *   k cache      [pages, page, Hkv, D] strides k_stride_page, k_stride_tok, k_stride_head
+ *   v cache      [pages, page, Hkv, Dv] strides v_stride_page, v_stride_tok, v_stride_head
+ *   o            [B, Hq, Dv]           strides o_stride_b, o_stride_h
  *   block_table  int32 [B, max_blocks] row stride bt_stride: physical page of logical page j
  *   kv_len       int32 [B]             context length; rows with kv_len <= 0 produce zeros
  * out[b, h] = softmax(q[b, h] . K[b, h / (Hq/Hkv)]^T * sm_scale) V, softmax in fp32 and P
@@ -138,14 +139,17 @@ int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t*
  * window_size > 0 masks keys older than kv_len - 1 - window_size (sliding window,
  * paged_attention.py:163-167,191-199); logit_softcapping > 0 replaces the scaled logits by
  * cap * tanh(logits / cap) (:186-189); pass <= 0 to disable either.
- * Supported: dtype bf16/f16, D in {64, 128}, page % 16 == 0, all strides multiples of 8 and
- * base pointers 16-byte aligned.  ws: dlb_paged_decode_ws_bytes(...) bytes of device scratch
- * (split-KV partials), caller-owned.
+ * Supported: dtype bf16/f16, key head size D and value head size Dv any multiples of 8 up to
+ * 128 (64 and 128 run the unmasked kernels; other sizes are computed in the next of those two
+ * with the extra dims masked, as the reference splits them into power-of-two blocks,
+ * kernels/paged_attention.py:531-539), page % 16 == 0, all strides multiples of 8 and base
+ * pointers 16-byte aligned.  ws: dlb_paged_decode_ws_bytes(B, Hq, Hkv, max(D, Dv), page,
+ * max_blocks) bytes of device scratch (split-KV partials), caller-owned.
  * ---------------------------------------------------------------------------------------- */
 size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int page, int max_blocks);
 int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, void* o,
                           const int32_t* block_table, const int32_t* kv_len, int B, int Hq,
-                          int Hkv, int D, int page, int max_blocks, int64_t q_stride_b,
+                          int Hkv, int D, int Dv, int page, int max_blocks, int64_t q_stride_b,
                           int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_tok,
                           int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_tok,
                           int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
@@ -163,9 +167,10 @@ int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cach
  * o[t, h] = sum_{t' <= t, same sequence} softmax_t'(q[t, h] . k[t', h / (Hq/Hkv)] * sm_scale)
  *           v[t', h / (Hq/Hkv)], softmax in fp32, P rounded to `dtype` before P.V.
  * (The reference fixes sm_scale = 1/sqrt(D); pass that for drop-in behaviour.)
- * Supported: dtype bf16/f16, D in {64, 128}, q/k/v strides multiples of 8 and bases 16-byte
- * aligned, o strides multiples of 4 and base 8-byte aligned.  Tokens outside every sequence
- * are not written.
+ * Supported: dtype bf16/f16, D any multiple of 8 up to 128 (the reference asserts
+ * D in {16, 32, 64, 128}, prefill_attention.py:160), q/k/v strides multiples of 8 and bases
+ * 16-byte aligned, o strides multiples of 4 and base 8-byte aligned.  Tokens outside every
+ * sequence are not written.
  * ---------------------------------------------------------------------------------------- */
 int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o,
                             const int32_t* start_loc, const int32_t* seq_len, int B, int Hq,
@@ -179,21 +184,24 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
  * their history (chunked prefill / prefix-cache hit), GQA.
  * Replaces the non-decoding branch of paged_attention_fwd + _fwd_kernel,
  * kernels/paged_attention.py:319-489, 559-607.
- *   q [tokens, Hq, D], o [tokens, Hq, D]: sequence s owns query tokens q_start_loc[s] ..
- *   q_start_loc[s] + q_len[s] - 1; k_cache/v_cache [pages, page, Hkv, D]; block_table int32
+ *   q [tokens, Hq, D], o [tokens, Hq, Dv]: sequence s owns query tokens q_start_loc[s] ..
+ *   q_start_loc[s] + q_len[s] - 1; k_cache [pages, page, Hkv, D], v_cache [pages, page, Hkv, Dv];
+ *   block_table int32
  *   [B, max_blocks]; kv_len int32 [B] = history + q_len[s] (sequences with kv_len < q_len are
  *   skipped).  Query i of sequence s sits at context position kv_len[s] - q_len[s] + i and
  *   sees keys 0 .. that position (paged_attention.py:455), or, with window_size > 0, only the
  *   keys >= position - window_size (:429-431,457-458); logit_softcapping > 0 replaces the
  *   scaled logits by cap * tanh(logits / cap) (:450-453).  Pass <= 0 to disable either.
  *   max_q_len >= max(q_len) sizes the grid.
- * Supported: dtype bf16/f16, D in {64, 128}, any page size >= 1, sm_scale > 0, q/k/v strides
- * multiples of 8 and bases 16-byte aligned, o strides multiples of 4 and base 8-byte aligned.
+ * Supported: dtype bf16/f16, D and Dv any multiples of 8 up to 128 (as for the decode entry
+ * point), any page size >= 1, sm_scale > 0, q/k/v strides multiples of 8 and bases 16-byte
+ * aligned, o strides multiples of 4 and base 8-byte aligned.
  * ---------------------------------------------------------------------------------------- */
 int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, void* o,
                            const int32_t* block_table, const int32_t* q_start_loc,
                            const int32_t* q_len, const int32_t* kv_len, int B, int Hq, int Hkv,
-                           int D, int page, int max_blocks, int max_q_len, int64_t q_stride_tok,
+                           int D, int Dv, int page, int max_blocks, int max_q_len,
+                           int64_t q_stride_tok,
                            int64_t q_stride_head, int64_t k_stride_page, int64_t k_stride_tok,
                            int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_tok,
                            int64_t v_stride_head, int64_t o_stride_tok, int64_t o_stride_head,

@@ -74,9 +74,10 @@ def gather_paged(cache, block_table_row, length):
 
 def paged_decode(q, k_cache, v_cache, block_table, kv_len, sm_scale=None, window=None,
                  softcap=None):
-    """q [B, Hq, D] -> o [B, Hq, D]; sequences with kv_len <= 0 give zeros."""
+    """q [B, Hq, D] -> o [B, Hq, Dv] (Dv = value head size of the cache); sequences with
+    kv_len <= 0 give zeros."""
     scale = sm_scale if sm_scale is not None else 1.0 / math.sqrt(q.shape[-1])
-    o = torch.zeros_like(q)
+    o = q.new_zeros((*q.shape[:-1], v_cache.shape[-1]))
     for b, length in enumerate(kv_len.tolist()):
         if length <= 0:
             continue
@@ -89,10 +90,10 @@ def paged_decode(q, k_cache, v_cache, block_table, kv_len, sm_scale=None, window
 def paged_prefill(q, k_cache, v_cache, block_table, q_start_loc, q_len, kv_len, sm_scale=None,
                   window=None, softcap=None):
     """q [T, Hq, D] packed; sequence b owns rows q_start_loc[b] .. + q_len[b], which are the
-    last q_len[b] of its kv_len[b] cached positions.  Returns o [T, Hq, D]; rows outside any
+    last q_len[b] of its kv_len[b] cached positions.  Returns o [T, Hq, Dv]; rows outside any
     sequence stay zero."""
     scale = sm_scale if sm_scale is not None else 1.0 / math.sqrt(q.shape[-1])
-    o = torch.zeros_like(q)
+    o = q.new_zeros((*q.shape[:-1], v_cache.shape[-1]))
     for b, (start, lq, lk) in enumerate(zip(q_start_loc.tolist(), q_len.tolist(), kv_len.tolist())):
         if lq <= 0 or lk < lq:
             continue
@@ -105,7 +106,7 @@ def paged_prefill(q, k_cache, v_cache, block_table, q_start_loc, q_len, kv_len, 
 
 
 def make_paged_cache(k_seqs, v_seqs, page, num_pages=None, seed=0, dtype=None):
-    """Scatter per-sequence K/V ([L_i, H, D] each) into a paged cache with pages assigned by
+    """Scatter per-sequence K ([L_i, H, D]) and V ([L_i, H, Dv]) into a paged cache with pages assigned by
     a seeded random permutation.  Returns (k_cache, v_cache, block_table int32 [B, max_blocks]).
     Unused table slots are 0; unused cache rows hold NaN so that any read past a context shows."""
     lens = [t.shape[0] for t in k_seqs]
@@ -115,9 +116,10 @@ def make_paged_cache(k_seqs, v_seqs, page, num_pages=None, seed=0, dtype=None):
     g = torch.Generator().manual_seed(seed)
     perm = torch.randperm(num_pages, generator=g)[:total].to(torch.int32)
     h, d = k_seqs[0].shape[1:]
+    dv = v_seqs[0].shape[2]
     dtype = dtype or k_seqs[0].dtype
     k_cache = torch.full((num_pages, page, h, d), float("nan"), dtype=dtype)
-    v_cache = torch.full((num_pages, page, h, d), float("nan"), dtype=dtype)
+    v_cache = torch.full((num_pages, page, h, dv), float("nan"), dtype=dtype)
     table = torch.zeros((len(lens), max(max(blocks), 1)), dtype=torch.int32)
     at = 0
     for b, (ks, vs) in enumerate(zip(k_seqs, v_seqs)):

@@ -12,7 +12,7 @@ def _rand(shape, seed, dtype):
 
 
 def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_dtype=torch.int32,
-              sm_scale=None, uniform=False, window=None, softcap=None):
+              sm_scale=None, uniform=False, window=None, softcap=None, dv=None):
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
     if uniform:   # the reference test draws torch.rand inputs (test_paged_attention.py:157-180)
@@ -21,13 +21,14 @@ def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_
     else:
         mk = lambda shape, s: _rand(shape, s, dtype)
     B = len(lens)
+    dv = dv or d
     ks = [mk((max(l, 1), hkv, d), 100 + i)[:l] for i, l in enumerate(lens)]
-    vs = [mk((max(l, 1), hkv, d), 200 + i)[:l] for i, l in enumerate(lens)]
+    vs = [mk((max(l, 1), hkv, dv), 200 + i)[:l] for i, l in enumerate(lens)]
     q = mk((B, hq, d), 7)
     kc, vc, table = oa.make_paged_cache(ks, vs, page, num_pages=num_pages, seed=seed, dtype=dtype)
     kv_len = torch.tensor(lens)
     ref = oa.paged_decode(q, kc, vc, table, kv_len, sm_scale=sm_scale, window=window, softcap=softcap)
-    o = torch.full((B, hq, d), 9.0, dtype=dtype, device=dev)
+    o = torch.full((B, hq, dv), 9.0, dtype=dtype, device=dev)
     ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(table_dtype).to(dev),
                               torch.arange(B, device=dev), torch.ones(B, dtype=torch.int64, device=dev),
                               kv_len.to(dev), 1, sm_scale=sm_scale, window_size=window,
@@ -41,13 +42,13 @@ def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_
 
 
 # the reference's own cases (test_paged_attention.py:244-255): decode rows seq_lens [1,1,1,1],
-# history [50,40,30,20], heads (8,2)/(2,2), page 16, fp16, uniform inputs; head dims moved to
-# the supported 64/128
+# history [50,40,30,20], heads (8,2)/(2,2), key head size 48/32 with value head size 32, page 16,
+# fp16, uniform inputs -- and the same at the unmasked sizes 64/128
 @pytest.mark.parametrize("hq,hkv", [(8, 2), (2, 2)])
-@pytest.mark.parametrize("d", [64, 128])
-def test_reference_decode_cases(dev, hq, hkv, d):
+@pytest.mark.parametrize("d,dv", [(48, 32), (32, 32), (64, 64), (128, 128)])
+def test_reference_decode_cases(dev, hq, hkv, d, dv):
     out, ref = _run_case(dev, [51, 41, 31, 21], hq, hkv, d, 16, torch.float16, uniform=True,
-                         table_dtype=torch.int64)
+                         table_dtype=torch.int64, dv=dv)
     # the reference's tolerance is atol 1e-3 on values in [0, 1]
     torch.testing.assert_close(out.float(), ref.float(), rtol=1e-5, atol=1e-3)
 
@@ -127,13 +128,16 @@ def test_strided_views(dev):
 def test_unsupported_requests_raise(dev):
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
-    q = torch.zeros((2, 4, 48), dtype=torch.float16, device=dev)
-    kc = torch.zeros((4, 16, 2, 48), dtype=torch.float16, device=dev)
-    o = torch.zeros_like(q)
-    args = (q, kc, kc, o, torch.zeros((2, 2), dtype=torch.int32, device=dev), None,
-            torch.ones(2, device=dev), torch.tensor([3, 4], device=dev), 1)
-    with pytest.raises(RuntimeError):
-        paged_attention_fwd(*args)                           # head dim 48
+    def args(d):
+        q = torch.zeros((2, 4, d), dtype=torch.float16, device=dev)
+        kc = torch.zeros((4, 16, 2, d), dtype=torch.float16, device=dev)
+        return (q, kc, kc, torch.zeros_like(q), torch.zeros((2, 2), dtype=torch.int32, device=dev),
+                None, torch.ones(2, device=dev), torch.tensor([3, 4], device=dev), 1)
+
+    with pytest.raises(NotImplementedError):
+        paged_attention_fwd(*args(44))                       # head size not a multiple of 8
+    with pytest.raises(NotImplementedError):
+        paged_attention_fwd(*args(136))                      # head size above 128
 
 
 def test_config4_full(dev):
@@ -166,3 +170,13 @@ def test_config4_full(dev):
     # whole-batch property: the output is a convex combination of V rows
     assert torch.isfinite(out.float()).all()
     assert out.float().abs().max() <= vc.float().abs().max()
+
+
+# head sizes that are not powers of two and value sizes that differ from the key size (the
+# reference splits them into power-of-two blocks, paged_attention.py:531-539)
+@pytest.mark.parametrize("d,dv", [(80, 80), (96, 96), (96, 64), (128, 64), (64, 128), (16, 8),
+                                  (120, 72), (40, 104)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_sizes(dev, d, dv, dtype):
+    _run_case(dev, [1, 17, 300, 1025, 64], 8, 2, d, 16, dtype, dv=dv, seed=d + dv)
+    _run_case(dev, [700, 33], 4, 4, d, 64, dtype, dv=dv, window=100, softcap=20.0)

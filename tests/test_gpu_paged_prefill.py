@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False, window=None,
-              softcap=None, sm_scale=None, max_seqlen=None, tol=2e-2):
+              softcap=None, sm_scale=None, max_seqlen=None, tol=2e-2, dv=None):
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
     gen = torch.Generator().manual_seed(123 + seed)
@@ -18,8 +18,9 @@ def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False,
     else:
         mk = lambda shape: torch.randn(shape, generator=gen).to(dtype)
     full = [a + b for a, b in zip(q_lens, hist)]
+    dv = dv or d
     ks = [mk((max(l, 1), hkv, d))[:l] for l in full]
-    vs = [mk((max(l, 1), hkv, d))[:l] for l in full]
+    vs = [mk((max(l, 1), hkv, dv))[:l] for l in full]
     T = sum(q_lens)
     q = mk((T + 3, hq, d))                                 # 3 rows owned by no sequence
     kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=seed, dtype=dtype)
@@ -27,7 +28,7 @@ def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False,
     ql, kl = torch.tensor(q_lens), torch.tensor(full)
     ref = oa.paged_prefill(q, kc, vc, table, start, ql, kl, sm_scale=sm_scale, window=window,
                            softcap=softcap)
-    o = torch.full((T + 3, hq, d), 9.0, dtype=dtype, device=dev)
+    o = torch.full((T + 3, hq, dv), 9.0, dtype=dtype, device=dev)
     ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(dev), start.to(dev),
                               ql.to(dev), kl.to(dev), max_seqlen or max(q_lens),
                               window_size=window, sm_scale=sm_scale, logit_softcapping=softcap)
@@ -40,21 +41,21 @@ def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False,
 
 
 # the reference's own prefill case (test_paged_attention.py:244-255): seq_lens [30,50,70,90]
-# after histories [50,40,30,20], heads (8,2)/(2,2), page 16, fp16, uniform inputs; head dims
-# moved to the supported 64/128
+# after histories [50,40,30,20], heads (8,2)/(2,2), key head size 48/32 with value head size 32,
+# page 16, fp16, uniform inputs -- and the same at the unmasked sizes 64/128
 @pytest.mark.parametrize("hq,hkv", [(8, 2), (2, 2)])
-@pytest.mark.parametrize("d", [64, 128])
-def test_reference_prefill_cases(dev, hq, hkv, d):
+@pytest.mark.parametrize("d,dv", [(48, 32), (32, 32), (64, 64), (128, 128)])
+def test_reference_prefill_cases(dev, hq, hkv, d, dv):
     out, ref = _run_case(dev, [30, 50, 70, 90], [50, 40, 30, 20], hq, hkv, d, 16, torch.float16,
-                         uniform=True)
+                         uniform=True, dv=dv)
     torch.testing.assert_close(out.float(), ref.float(), rtol=1e-5, atol=1e-3)
 
 
 # the reference's window case (test_paged_attention.py:291-303): window 32 on the same lengths
-@pytest.mark.parametrize("d", [64, 128])
-def test_reference_window_case(dev, d):
+@pytest.mark.parametrize("d,dv", [(48, 32), (64, 64), (128, 128)])
+def test_reference_window_case(dev, d, dv):
     out, ref = _run_case(dev, [30, 50, 70, 90], [50, 40, 30, 20], 4, 2, d, 16, torch.float16,
-                         uniform=True, window=32)
+                         uniform=True, window=32, dv=dv)
     torch.testing.assert_close(out.float(), ref.float(), rtol=1e-5, atol=1e-3)
 
 
@@ -117,9 +118,9 @@ def test_grid_larger_than_needed_and_rejects(dev):
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
     _run_case(dev, [10, 20], [5, 0], 2, 2, 64, 16, torch.float16, max_seqlen=1000)
-    q = torch.zeros(8, 2, 96, dtype=torch.float16, device=dev)          # unsupported head dim
-    kc = torch.zeros(4, 16, 2, 96, dtype=torch.float16, device=dev)
-    with pytest.raises(_lib.DlblasHipError):
+    q = torch.zeros(8, 2, 100, dtype=torch.float16, device=dev)         # head size not a multiple of 8
+    kc = torch.zeros(4, 16, 2, 100, dtype=torch.float16, device=dev)
+    with pytest.raises(NotImplementedError):
         paged_attention_fwd(q, kc, kc, torch.empty_like(q), torch.zeros(2, 2, dtype=torch.int32, device=dev),
                             torch.tensor([0, 4], device=dev), torch.tensor([4, 4], device=dev),
                             torch.tensor([4, 4], device=dev), 4)
@@ -135,3 +136,11 @@ def test_many_sequences_any_order(dev, nseq):
     hist = torch.randint(0, 40, (nseq,), generator=g).tolist()
     hist[1] = hist[0] + q_lens[0] - q_lens[1] if hist[0] + q_lens[0] >= q_lens[1] else hist[1]
     _run_case(dev, q_lens, hist, 4, 2, 128, 16, torch.bfloat16, seed=nseq)
+
+
+# head sizes that are not powers of two and value sizes that differ from the key size
+@pytest.mark.parametrize("d,dv", [(80, 80), (96, 64), (128, 64), (64, 128), (16, 8), (120, 72)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_sizes(dev, d, dv, dtype):
+    _run_case(dev, [1, 130, 64, 33], [0, 300, 64, 7], 8, 2, d, 16, dtype, dv=dv, seed=d + dv)
+    _run_case(dev, [200], [1000], 4, 4, d, 48, dtype, dv=dv, window=150, softcap=25.0)

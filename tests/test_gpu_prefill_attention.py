@@ -131,3 +131,11 @@ def test_config3_full(dev):
     # every first token of a sequence must reproduce its own V row exactly
     for b in range(8):
         assert torch.equal(out[int(cu[b])], v[int(cu[b])].repeat_interleave(4, dim=0))
+
+
+# the head sizes the reference's wrapper accepts (prefill_attention.py:160: 16, 32, 64, 128) and
+# sizes in between; 64 and 128 run the unmasked kernels, the others the masked variants
+@pytest.mark.parametrize("d", [16, 32, 48, 80, 96, 120])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_sizes(dev, d, dtype):
+    _run(dev, [1, 33, 64, 129, 700], 8, 2, d, dtype, gap=2)

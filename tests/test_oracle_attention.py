@@ -151,3 +151,38 @@ def test_paged_prefill_window():
             row = oa.paged_decode(q[start[b] + i][None], kc, vc, table[b][None], torch.tensor([ctx]),
                                   window=8)
             assert torch.equal(out[start[b] + i], row[0])
+
+
+def test_value_head_size_may_differ_from_key_head_size():
+    # the reference's own paged-attention matrix runs key size 48 / 32 with value size 32
+    # (test_paged_attention.py:244-246); pinned here by torch's SDPA on the gathered context
+    g = torch.Generator().manual_seed(21)
+    lens = [37, 5, 64]
+    hq, hkv, dk, dv, page = 4, 2, 48, 32, 16
+    ks = [torch.randn((l, hkv, dk), generator=g) for l in lens]
+    vs = [torch.randn((l, hkv, dv), generator=g) for l in lens]
+    q = torch.randn((len(lens), hq, dk), generator=g)
+    kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=1)
+    assert kc.shape[-1] == dk and vc.shape[-1] == dv
+    out = oa.paged_decode(q, kc, vc, table, torch.tensor(lens))
+    assert out.shape == (len(lens), hq, dv)
+    for b, l in enumerate(lens):
+        kk = ks[b].transpose(0, 1).repeat_interleave(hq // hkv, 0)
+        vv = vs[b].transpose(0, 1).repeat_interleave(hq // hkv, 0)
+        ref = torch.nn.functional.scaled_dot_product_attention(q[b][:, None, :], kk, vv)[:, 0]
+        torch.testing.assert_close(out[b], ref, rtol=1e-5, atol=1e-5)
+    # prefill with history: every query row equals a decode over the context ending at it
+    q_lens, hist = [7, 3], [11, 0]
+    full = [a + b for a, b in zip(q_lens, hist)]
+    ks = [torch.randn((l, hkv, dk), generator=g) for l in full]
+    vs = [torch.randn((l, hkv, dv), generator=g) for l in full]
+    kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=2)
+    qp = torch.randn((sum(q_lens), hq, dk), generator=g)
+    start = torch.tensor([0, q_lens[0]])
+    o = oa.paged_prefill(qp, kc, vc, table, start, torch.tensor(q_lens), torch.tensor(full))
+    assert o.shape == (sum(q_lens), hq, dv)
+    for b in range(2):
+        for i in range(q_lens[b]):
+            row = start[b].item() + i
+            one = oa.paged_decode(qp[row][None], kc, vc, table[b][None], torch.tensor([hist[b] + i + 1]))
+            torch.testing.assert_close(o[row], one[0], rtol=1e-5, atol=1e-5)
