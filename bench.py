@@ -413,7 +413,7 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         lib = _lib.load()
         block = fm._BLOCK_M
         sorted_ids, _, _, counts = moe_align_block_size(ids, block, E, return_counts=True)
-        nmb = -(-sorted_ids.numel() // block)
+        nmb = sorted_ids.numel() // block
         xq, xs = fm.per_token_group_quant_fp8(x)
         hq = torch.empty((nmb * block, I), dtype=torch.float8_e4m3fn, device=dev)
         hs = torch.empty((nmb * block, I // 128), dtype=torch.float32, device=dev)

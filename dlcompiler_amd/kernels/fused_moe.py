@@ -121,7 +121,7 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     block = _BLOCK_M
     sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
                                                     return_counts=True)
-    num_mblocks = -(-sorted_ids.numel() // block)
+    num_mblocks = sorted_ids.numel() // block  # whole blocks the slot list can hold
     xq, xs = per_token_group_quant_fp8(hidden_states)
 
     # one allocation for the intermediates: fp8 rows + their scales (fp32) + the slot outputs
@@ -194,7 +194,7 @@ def fused_moe(hidden_states: torch.Tensor,
     block = _BLOCK_M
     sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
                                                     return_counts=True)
-    num_mblocks = -(-sorted_ids.numel() // block)
+    num_mblocks = sorted_ids.numel() // block  # whole blocks the slot list can hold
     act = torch.empty((num_mblocks * block, I), dtype=dt, device=dev)
     full = (expert_offset == 0 and num_experts == E)
     slots = (torch.empty if full else torch.zeros)((M * topk, O), dtype=dt, device=dev)

@@ -230,8 +230,11 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
  *   sorted_ids [num_mblocks * block_m] and expert_counts [num_experts]: the sorted slot list and
  *     the per-expert counts written by dlb_moe_align_block_size with block = block_m over all
  *     num_experts (global) experts; block_m in {64, 128} = rows per workgroup tile; flat slot =
- *     token * topk + j, sentinel num_tokens * topk.  num_mblocks = capacity of sorted_ids in
- *     blocks (>= sum over experts of ceil(count / block_m)).  Expert e's blocks start at block
+ *     token * topk + j, sentinel num_tokens * topk.  num_mblocks = whole blocks sorted_ids
+ *     holds (it has at least num_mblocks * block_m entries; floor(sorted_cap / block_m) of the
+ *     alignment call is always >= sum over experts of ceil(count / block_m), the blocks in use;
+ *     a workgroup whose block index is not below num_mblocks touches nothing).  Expert e's
+ *     blocks start at block
  *     sum_{e' < e} ceil(count[e'] / block_m); blocks of experts outside
  *     [expert_offset, expert_offset + num_local_experts) are skipped.  num_experts <= 256.
  *   hq [num_mblocks * block_m, I] fp8 and hs [num_mblocks * block_m, I/128]: row r holds

@@ -60,3 +60,23 @@ def test_argument_validation_needs_no_gpu():
     assert lib.dlb_moe_topk_softmax_f32(None, None, None, 4, 64, 65, 64, 1, None) == -1
     assert lib.dlb_moe_topk_softmax_f32(None, None, None, 4, 512, 2, 512, 1, None) == -2
     assert lib.dlb_moe_align_ws_bytes(98304, 64) > 0
+
+
+def test_moe_gemm_argument_checks_need_no_gpu():
+    # the grouped-GEMM entry points validate on the host; nothing is launched for a bad request
+    lib = _lib.load()
+    one = 16  # any non-null, 16-byte aligned fake pointer: rejected before it is dereferenced
+
+    def gate_up(num_experts=8, num_mblocks=4, block_m=128, H=256, I=128, offset=0, local=8):
+        return lib.dlb_moe_gemm_fp8_gate_up(one, one, one, one, one, one, num_experts, num_mblocks,
+                                            block_m, 64, 2, H, I, offset, local, 1, one, one, None)
+
+    assert gate_up(num_mblocks=0) == 0                    # nothing to do
+    assert gate_up(block_m=96) == -2                      # tile heights are 64 and 128
+    assert gate_up(H=200) == -2                           # rows are whole 128-byte chunks
+    assert gate_up(num_experts=300, local=300) == -2      # at most 256 experts
+    assert gate_up(offset=4, local=8) == -1               # local experts must lie inside the global range
+    assert gate_up(num_mblocks=-1) == -1
+    assert lib.dlb_moe_gemm_fp8_gate_up(one, one, one, one, one, None, 8, 4, 128, 64, 2, 256, 128,
+                                        0, 8, 1, one, one, None) == -1   # counts are required
+    assert lib.dlb_moe_align_block_size_static_max_numel() == 256 * 2048

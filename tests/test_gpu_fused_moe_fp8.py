@@ -202,3 +202,20 @@ def test_fused_moe_fp8_repeats_bit_identically(dev, block, monkeypatch):
     # both weight layouts hold the same numbers: same result
     plain = fm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids, k, weights_shuffled=False)
     assert torch.equal(plain, first)
+
+
+@pytest.mark.parametrize("out_size", [128, 384])
+def test_output_width_comes_from_w2(dev, out_size):
+    # the reference sizes the result from w2.shape[1] (fused_moe.py:354-357): it need not be H
+    from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8
+
+    T, H, I, E, k = 150, 256, 256, 4, 2
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn((T, H), generator=g).bfloat16()
+    tw, ids = og.topk_softmax(torch.randn((T, E), generator=g), k, renormalize=True)
+    w1q, w1s = ofp8.block_quant_weight(torch.randn((E, 2 * I, H), generator=g) * 0.05)
+    w2q, w2s = ofp8.block_quant_weight(torch.randn((E, out_size, I), generator=g) * 0.05)
+    ref = ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids)
+    out = fused_moe_fp8(*[t.to(dev) for t in (x, w1q, w1s, w2q, w2s, tw, ids)], k)
+    assert out.shape == (T, out_size)
+    _check(out.cpu(), ref)
