@@ -91,7 +91,7 @@ def _time_steps(step, steps, warmup):
     stats: STAT_ITERS further iterations in STAT_BATCHES batches, one event pair per batch; the
     median / p10 / p90 are over the per-step times of the batches (batch time / batch size).  For
     a single-kernel workload a step is that kernel's launch, launch gaps included."""
-    for i in range(max(warmup, MIN_WARMUP)):
+    for i in range(warmup if COUNTER_PASS else max(warmup, MIN_WARMUP)):
         step(i)
     torch.cuda.synchronize()
     t_all = Timer()
@@ -104,7 +104,12 @@ def _time_steps(step, steps, warmup):
     return ms, _batch_stats(step)
 
 
-def _batch_stats(step, iters=STAT_ITERS, batches=STAT_BATCHES):
+COUNTER_PASS = False  # --counters: a run under a hardware-counter pass keeps launches few
+
+
+def _batch_stats(step, iters=None, batches=None):
+    iters = iters or (4 if COUNTER_PASS else STAT_ITERS)
+    batches = batches or (2 if COUNTER_PASS else STAT_BATCHES)
     per = max(1, -(-iters // batches))
     tb = Timer()
     n = 0
@@ -191,6 +196,8 @@ def wl_silu(dev, steps, warmup, cpu):
 
 
 def _graph_replay_ms(fn, steps, warmup, label):
+    if COUNTER_PASS:
+        return None
     """Mean time of one replay of ``fn`` captured into a HIP graph (optional extra figure: the
     public calls with no Python or launch latency between their kernels).  None if capture fails."""
     try:
@@ -685,7 +692,13 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first launch an elementwise copy of 1 GiB (fp32 x * 1 -> y) three times: "
                          "the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--counters", action="store_true",
+                    help="for a run under rocprofv3 --pmc, where every launch is serialised: "
+                         "--warmup is taken as given, 4 statistics iterations instead of "
+                         f"{STAT_ITERS}, no graph replays; the timings of such a run mean nothing")
     args = ap.parse_args()
+    global COUNTER_PASS
+    COUNTER_PASS = args.counters
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the operators are single-device; "
               "no collective is part of the path) -- run with --gpus 1", file=sys.stderr)

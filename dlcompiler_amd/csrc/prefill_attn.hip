@@ -15,7 +15,10 @@
 //     from ds_read_b64_tr_b16, which hands lane l of a 16-lane group column l of a 4-row x
 //     16-column block (rows supplied by lanes 4j .. 4j+3), i.e. the transpose happens in the
 //     LDS read and V never passes through registers on its way in;
-//   * the exponent runs in base 2 with the softmax scale folded into one FMA;
+//   * the exponent runs in base 2: Q is multiplied by scale * log2(e) once when it is loaded, and
+//     the score accumulators start at minus the running reference, so the MFMAs deliver the
+//     argument of exp2 and the softmax costs one maximum, one exponential and one addition per
+//     score;
 //   * fully masked tiles are skipped per wave and only diagonal tiles pay for the mask; the
 //     heaviest query tiles are launched first.
 #include <type_traits>
@@ -63,6 +66,10 @@ struct Mma32<DLB_DTYPE_BF16> {
     f2 f = {a, b};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, b2));
   }
+  // both elements of a packed pair times c, rounded back to the element type
+  static __device__ __forceinline__ unsigned int scale2(unsigned int w, float c) {
+    return pack2(__uint_as_float(w << 16) * c, __uint_as_float(w & 0xffff0000u) * c);
+  }
 };
 template <>
 struct Mma32<DLB_DTYPE_F16> {
@@ -75,6 +82,12 @@ struct Mma32<DLB_DTYPE_F16> {
     typedef __attribute__((ext_vector_type(2))) _Float16 h2;
     f2 f = {a, b};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, h2));
+  }
+  static __device__ __forceinline__ unsigned int scale2(unsigned int w, float c) {
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    const f2 f = __builtin_convertvector(__builtin_bit_cast(h2, w), f2);
+    return pack2(f[0] * c, f[1] * c);
   }
 };
 
@@ -110,11 +123,11 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   // between the sequences of a batch while the grid holds only a few workgroups per slot, so
   // the sequences are walked longest context first (blockIdx.z = rank, not index): the long
   // ones start in the first round and the short ones fill in behind them.
-  // Packed layout: a tile's cost is set by its position in its sequence alone, so the grid runs
-  // over (head, sequence, query tile) with the tile index slowest and reversed: the last tiles
-  // of the long sequences start first, everywhere, and the cheap first tiles of all sequences
-  // finish the launch.
-  int seq = PAGED ? blockIdx.z : blockIdx.y;
+  // Both layouts run the grid over (head, query tile, sequence), tile index reversed: what an
+  // XCD holds at any time is the query tiles of ONE sequence's heads of ONE KV group (see the head
+  // remap below), i.e. workgroups that stream the same K/V rows, which its L2 then serves after
+  // the first read; within a sequence the heaviest (last) tiles start first.
+  int seq = blockIdx.z;
   if (PAGED && gridDim.z > 1 && gridDim.z <= kThreads) {
     __shared__ int32_t rank_key[kThreads];
     __shared__ int32_t rank_seq;
@@ -135,7 +148,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     seq = __builtin_amdgcn_readfirstlane(rank_seq);
   }
   const int L = p.seq_len[seq];
-  const int qtile = PAGED ? gridDim.y - 1 - blockIdx.y : gridDim.z - 1 - blockIdx.z;  // heaviest first
+  const int qtile = gridDim.y - 1 - blockIdx.y;  // heaviest first
   const int q0 = qtile * kBlockM;
   if (q0 >= L) return;
   const int64_t tok0 = p.start_loc[seq];
@@ -157,7 +170,9 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   const unsigned short* kb = (const unsigned short*)p.k + (int64_t)kvh * p.k_sh;
   const unsigned short* vb = (const unsigned short*)p.v + (int64_t)kvh * p.v_sh;
 
-  // ---- Q^T as B operand: lane (n = query, k = dims 16*ks + 8*hh .. +8), kept in registers
+  // ---- Q^T as B operand: lane (n = query, k = dims 16*ks + 8*hh .. +8), kept in registers,
+  // multiplied once by scale * log2(e) (and rounded back to the element type) so that the score
+  // MFMAs deliver exponents of 2 directly
   const int qrow = q0 + 32 * wave + col;
   u32x4 qf[KS];
   {
@@ -167,6 +182,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     for (int ks = 0; ks < KS; ++ks) {
       qf[ks] = u32x4{0u, 0u, 0u, 0u};
       if (!RAGGED || 16 * ks + 8 * hh < p.dk) qf[ks] = *(const u32x4*)(qp + 16 * ks);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) qf[ks][w] = Mma32<DT>::scale2(qf[ks][w], p.scale_log2e);
     }
   }
 
@@ -297,10 +314,15 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   // lazily: the accumulators are rescaled only when a row maximum exceeds it by more than
   // kRescaleGap, so between rescales probabilities stay below 2^kRescaleGap -- exact in the
   // end (the same factor cancels in O / l), and it removes the per-tile rescale of O.
+  // The reference is not subtracted by vector instructions: the score accumulators START at
+  // -m_run (neg_ref, the C operand of the first k-step), so the MFMAs deliver s - m_run and the
+  // exponential is the only per-score instruction besides the maximum and the sum.
   constexpr float kRescaleGap = 8.0f;
-  float m_run = -__builtin_inff();
+  float m_run = -__builtin_inff();  // -inf: no visible key seen yet (the accumulators then start at 0)
   float l_run = 0.0f;  // this lane half's share of the denominator
-  const float cs = p.scale_log2e;
+  f32x16 neg_ref;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) neg_ref[i] = 0.0f;
 
   // byte offsets of this lane's transposing V reads inside a tile, one per 32-dim block
   int v_off[MT];
@@ -330,10 +352,6 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     // k-step outer, key tile inner: two independent accumulator chains, and the K fragments
     // are fetched from LDS two k-steps ahead of the MFMAs that consume them
     f32x16 s[2];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
     // MFMA-dense phase: let this wave's issue win over the other wave of the SIMD, whose
     // softmax arithmetic then fills the gaps while the matrix pipe is busy
     __builtin_amdgcn_s_setprio(1);
@@ -355,14 +373,15 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         if (kstep + kAhead < KS) ldk(kstep + kAhead, ka[(kstep + kAhead) % (kAhead + 1)]);
         if (COPY) issue_copy(kstep);
         __builtin_amdgcn_sched_barrier(0);  // keep the fetch ahead of the MFMAs (it would be sunk)
-        s[0] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][0], qf[kstep], s[0]);
-        s[1] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][1], qf[kstep], s[1]);
+        s[0] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][0], qf[kstep], kstep == 0 ? neg_ref : s[0]);
+        s[1] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][1], qf[kstep], kstep == 0 ? neg_ref : s[1]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
 
     __builtin_amdgcn_s_setprio(0);
-    // ---- causal mask and tile maximum of the raw scores (scale > 0 commutes with max)
+    // ---- causal mask and tile maximum of the scores, which arrive relative to the reference
+    const float m_ref = (m_run == -__builtin_inff()) ? 0.0f : m_run;  // what neg_ref holds, negated
     float mpart[2] = {-__builtin_inff(), -__builtin_inff()};  // two independent chains
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
@@ -371,8 +390,10 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         if (MASK) {
           const int key = t0 + 32 * nt + 8 * (i >> 2) + 4 * hh + (i & 3);
           float x = s[nt][i];
-          if (softcap > 0.0f)  // cap * tanh(x * scale / cap), kept in raw-score units
-            x = tanhf(x * (p.sm_scale / softcap)) * (softcap / p.sm_scale);
+          if (softcap > 0.0f) {  // cap * tanh(score * scale / cap), all in log2 units
+            const float cap2 = softcap * 1.4426950408889634f;
+            x = tanhf((x + m_ref) / cap2) * cap2 - m_ref;
+          }
           bool vis = key <= qpos;
           if (window > 0) vis = vis && (key >= qpos - window);
           s[nt][i] = vis ? x : -__builtin_inff();
@@ -380,26 +401,36 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         mpart[nt] = fmaxf(mpart[nt], s[nt][i]);
       }
     }
-    const float mloc = max_xor32(fmaxf(mpart[0], mpart[1])) * cs;
-    if (__any(mloc > m_run + kRescaleGap)) {
-      const float m_new = fmaxf(m_run, mloc);  // finite from tile 0 on (key 0 is visible)
-      // (a fully masked row under a sliding window keeps m_new = -inf: leave it untouched)
-      const float alpha = (MASK && PAGED && m_new == -__builtin_inff()) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-      m_run = m_new;
+    const float mloc = max_xor32(fmaxf(mpart[0], mpart[1]));  // relative to the reference
+    const bool unset = m_run == -__builtin_inff();
+    // the reference moves when a row maximum exceeds it by more than the gap, and is set by the
+    // first tile that shows the row a visible key (whatever its sign: it may lie far below 0)
+    if (__any(mloc > kRescaleGap || (unset && mloc > -__builtin_inff()))) {
+      // rows still without a visible key stay unset; rows that are set only move up
+      const float delta = unset ? mloc : fmaxf(mloc, 0.0f);  // -inf only for rows that stay unset
+      const bool stay = unset && mloc == -__builtin_inff();
+      const float d = stay ? 0.0f : delta;
+      const float alpha = unset ? 1.0f : __builtin_amdgcn_exp2f(-d);  // o and l are 0 while unset
+      if (!stay) m_run = m_ref + d;
       l_run *= alpha;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
+      const float nr = stay ? 0.0f : -m_run;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) neg_ref[i] = nr;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[nt][i] -= d;
     }
-    // a row whose keys so far were all masked (sliding window) still has m_run = -inf
-    const float m_ref = (MASK && PAGED && m_run == -__builtin_inff()) ? 0.0f : m_run;
     float psum = 0.0f;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][i], cs, -m_ref));
+        const float e = __builtin_amdgcn_exp2f(s[nt][i]);
         s[nt][i] = e;
         psum += e;
       }
@@ -505,7 +536,7 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk,
     if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
   if (p.o_st % 4 != 0 || p.o_sh % 4 != 0) return DLB_ERR_UNSUPPORTED;
   if (B > 65535) return DLB_ERR_UNSUPPORTED;
-  if (!(sm_scale > 0.0f)) return DLB_ERR_BAD_ARG;  // the tile maximum is taken before scaling
+  if (!(sm_scale > 0.0f)) return DLB_ERR_BAD_ARG;
 
   p.Hq = Hq;
   p.Hkv = Hkv;
@@ -520,7 +551,7 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk,
   hipStream_t s = (hipStream_t)stream;
   const uint32_t qtiles = (uint32_t)ceil_div(max_len, kBlockM);
   if (qtiles > 65535) return DLB_ERR_UNSUPPORTED;
-  const dim3 grid = paged ? dim3((uint32_t)Hq, qtiles, (uint32_t)B) : dim3((uint32_t)Hq, (uint32_t)B, qtiles);
+  const dim3 grid = dim3((uint32_t)Hq, qtiles, (uint32_t)B);
 #define DLB_LAUNCH_PREFILL(DT_, D_, PG_)                                                          \
   do {                                                                                            \
     if (ragged)                                                                                   \
