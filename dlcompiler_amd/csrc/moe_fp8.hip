@@ -250,20 +250,21 @@ __device__ __forceinline__ bool find_tile(const MoeGemmParams& p, int lane, Tile
 // chunks of weights and two fragment buffers fit the 256 registers of a wave at two waves per
 // SIMD.  (Scales are floored at 1e-30 so that a zero scale cannot divide.)
 //
-// Data movement, all of it issued by hand so that nothing waits for more than it needs (the
-// compiler's wait-count pass treats a load under a run-time condition as possibly absent and
-// then waits for everything younger too, which defeats a deep prefetch):
-//   * weights: global -> operand registers in units of (chunk half, both column tiles) = 4 x 16
-//     bytes per lane; a ring of four units (two chunks), each refilled right after its last
-//     use for the chunk after next (1.5 chunks ahead);
-//   * activations: global -> LDS directly (three chunk slots of 128 x 128 bytes, rows swizzled
-//     by (row >> 1) & 7 in 16-byte pieces), wave w stages row tile w, issued two chunks ahead;
-//     one barrier per chunk, between its two halves, publishes the next chunk; the scales of a
-//     chunk travel with it (one 4-byte copy per wave: the activation scales of its 32 staging
-//     rows and its own two block scales);
-//   * every wave issues the same number of loads per chunk (chunks past K re-load clamped or
-//     dummy addresses, waves whose row tile is padding copy one dummy line), so the explicit
-//     vmcnt waits are compile-time constants.
+// Data movement:
+//   * weights: global -> operand registers with plain loads, in units of (chunk half, both
+//     column tiles) = 4 x 16 bytes per lane; two chunks of units live in registers, each unit
+//     re-loaded right after its last use for the chunk after next (1.5 chunks ahead).  The
+//     compiler owns these registers and places their waits (issued from inline assembly the
+//     four pieces of a unit do not end up in adjacent registers, and the copies that gather
+//     them cost more than the exact waits save);
+//   * activations: global -> LDS directly, by hand (three chunk slots of 128 x 128 bytes, rows
+//     swizzled by (row >> 1) & 7 in 16-byte pieces), wave w stages row tile w, issued two chunks
+//     ahead; one barrier per chunk, between its two halves, publishes the next chunk; the
+//     activation scales of a chunk travel with it (one 4-byte copy per wave).  The compiler does
+//     not see these copies, so the kernel waits for them itself with a constant vmcnt: every
+//     wave issues the same number of vector-memory operations per chunk (chunks past K re-load
+//     clamped addresses, waves whose row tile is padding copy one dummy line);
+//   * the block scales of the wave's two column tiles are parked in LDS once per tile.
 // None of this may go through scratch memory: the build checks that the kernel spills nothing.
 template <bool GATED, int DT, int QT, int WL>
 __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p) {
