@@ -119,14 +119,15 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
 
   __shared__ __attribute__((aligned(16))) unsigned char smem[2 * SM::stage];
 
+  // The grid runs over (head, query tile, sequence), tile index reversed: what an XCD holds at
+  // any time is the query tiles of ONE sequence's heads of ONE KV group (see the head remap
+  // below), i.e. workgroups that stream the same K/V rows, which its L2 then serves after the
+  // first read; within a sequence the heaviest (last) tiles start first.
   // Paged (chunked) prefill: a sequence's cost is set by its history, which differs widely
   // between the sequences of a batch while the grid holds only a few workgroups per slot, so
   // the sequences are walked longest context first (blockIdx.z = rank, not index): the long
-  // ones start in the first round and the short ones fill in behind them.
-  // Both layouts run the grid over (head, query tile, sequence), tile index reversed: what an
-  // XCD holds at any time is the query tiles of ONE sequence's heads of ONE KV group (see the head
-  // remap below), i.e. workgroups that stream the same K/V rows, which its L2 then serves after
-  // the first read; within a sequence the heaviest (last) tiles start first.
+  // ones start in the first round and the short ones fill in behind them.  (The packed layout
+  // has many workgroups per slot and gains nothing from the ranking: measured 1.5 % slower.)
   int seq = blockIdx.z;
   if (PAGED && gridDim.z > 1 && gridDim.z <= kThreads) {
     __shared__ int32_t rank_key[kThreads];
