@@ -161,6 +161,47 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(
   }
 }
 
+// fp32 rows: the same kernel shape on four-element vectors (nothing is rounded on the way, so
+// the two rounding points above coincide).
+constexpr int kMaxVecF32 = 16;  // 256 threads * 16 vectors * 4 elements = 16384 columns
+template <bool ADD>
+__global__ __launch_bounds__(kNormThreads) void rms_norm_f32_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ res,
+    float* __restrict__ out, float* __restrict__ out_res, int N, int64_t ld_x, int64_t ld_res,
+    int64_t ld_out, int64_t ld_out_res, float eps) {
+  __shared__ float red[kNormThreads / 64];
+  const int64_t row = blockIdx.x;
+  const int nvec = N >> 2;
+  f32x4 v[kMaxVecF32];
+  float ss = 0.0f;
+#pragma unroll
+  for (int q = 0; q < kMaxVecF32; ++q) {
+    const int i = q * kNormThreads + threadIdx.x;
+    if (i < nvec) {
+      v[q] = __builtin_nontemporal_load((const f32x4*)(x + row * ld_x + 4 * i));
+      if (ADD) {
+        v[q] += __builtin_nontemporal_load((const f32x4*)(res + row * ld_res + 4 * i));
+        __builtin_nontemporal_store(v[q], (f32x4*)(out_res + row * ld_out_res + 4 * i));
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) ss += v[q][k] * v[q][k];
+    }
+  }
+  const float var = block_sum(ss, red) / (float)N;
+  const float inv = rsqrtf(var + eps);
+#pragma unroll
+  for (int q = 0; q < kMaxVecF32; ++q) {
+    const int i = q * kNormThreads + threadIdx.x;
+    if (i < nvec) {
+      const f32x4 wv = *(const f32x4*)(w + 4 * i);
+      f32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = (v[q][k] * inv) * wv[k];
+      __builtin_nontemporal_store(o, (f32x4*)(out + row * ld_out + 4 * i));
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // rotary: for d < D/2:  out[d]       = x[d] * cos[d]       - x[d + D/2] * sin[d]
 //                       out[d + D/2] = x[d + D/2] * cos[d + D/2] + x[d] * sin[d + D/2]
@@ -208,6 +249,44 @@ __global__ __launch_bounds__(256) void rotary_kernel(
     }
     __builtin_nontemporal_store(ol, (u32x4*)(dst + 8 * c));
     __builtin_nontemporal_store(oh, (u32x4*)(dst + half + 8 * c));
+  }
+}
+
+// fp32 tensors: a thread handles 4 low and the 4 matching high elements of one head
+__global__ __launch_bounds__(256) void rotary_f32_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ cos_,
+    const float* __restrict__ sin_, float* qo, float* ko, int Hq, int Hk, int D, int64_t q_st,
+    int64_t q_sh, int64_t k_st, int64_t k_sh, int64_t qo_st, int64_t qo_sh, int64_t ko_st,
+    int64_t ko_sh, int64_t cs_st) {
+  const int64_t t = blockIdx.x;
+  const int half = D >> 1;
+  const int vec_per_head = half >> 2;
+  const int total = (Hq + Hk) * vec_per_head;
+  for (int u = threadIdx.x; u < total; u += 256) {
+    const int h = u / vec_per_head, c = u - h * vec_per_head;
+    const float* src;
+    float* dst;
+    if (h < Hq) {
+      src = q + t * q_st + (int64_t)h * q_sh;
+      dst = qo + t * qo_st + (int64_t)h * qo_sh;
+    } else {
+      src = k + t * k_st + (int64_t)(h - Hq) * k_sh;
+      dst = ko + t * ko_st + (int64_t)(h - Hq) * ko_sh;
+    }
+    const f32x4 xl = __builtin_nontemporal_load((const f32x4*)(src + 4 * c));
+    const f32x4 xh = __builtin_nontemporal_load((const f32x4*)(src + half + 4 * c));
+    const f32x4 cl = *(const f32x4*)(cos_ + t * cs_st + 4 * c);
+    const f32x4 ch = *(const f32x4*)(cos_ + t * cs_st + half + 4 * c);
+    const f32x4 sl = *(const f32x4*)(sin_ + t * cs_st + 4 * c);
+    const f32x4 sh = *(const f32x4*)(sin_ + t * cs_st + half + 4 * c);
+    f32x4 ol, oh;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ol[j] = xl[j] * cl[j] - xh[j] * sl[j];
+      oh[j] = xh[j] * ch[j] + xl[j] * sh[j];
+    }
+    __builtin_nontemporal_store(ol, (f32x4*)(dst + 4 * c));
+    __builtin_nontemporal_store(oh, (f32x4*)(dst + half + 4 * c));
   }
 }
 
@@ -281,16 +360,30 @@ extern "C" int dlb_rms_norm(const void* x, const void* weight, const void* resid
   if (M < 0 || N < 1) return DLB_ERR_BAD_ARG;
   if (M == 0) return DLB_OK;
   if (!x || !weight || !out || (residual && !out_residual)) return DLB_ERR_BAD_ARG;
-  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
-  if (N % 8 != 0 || N > kNormThreads * kMaxVec * 8) return DLB_ERR_UNSUPPORTED;
-  if (ld_x % 8 != 0 || ld_out % 8 != 0 || !aligned16(x) || !aligned16(weight) || !aligned16(out))
+  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16 && dtype != DLB_DTYPE_F32)
     return DLB_ERR_UNSUPPORTED;
-  if (residual && (ld_res % 8 != 0 || ld_out_res % 8 != 0 || !aligned16(residual) ||
+  const int vec = dtype == DLB_DTYPE_F32 ? 4 : 8;  // elements per 16-byte vector
+  if (N % vec != 0 || N > kNormThreads * kMaxVec * 8) return DLB_ERR_UNSUPPORTED;
+  if (ld_x % vec != 0 || ld_out % vec != 0 || !aligned16(x) || !aligned16(weight) || !aligned16(out))
+    return DLB_ERR_UNSUPPORTED;
+  if (residual && (ld_res % vec != 0 || ld_out_res % vec != 0 || !aligned16(residual) ||
                    !aligned16(out_residual)))
     return DLB_ERR_UNSUPPORTED;
   if (M > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)M), block(kNormThreads);
+  static_assert(kMaxVecF32 * 4 == kMaxVec * 8, "same row length limit for every element type");
+  if (dtype == DLB_DTYPE_F32) {
+    if (residual)
+      hipLaunchKernelGGL(rms_norm_f32_kernel<true>, grid, block, 0, s, (const float*)x,
+                         (const float*)weight, (const float*)residual, (float*)out,
+                         (float*)out_residual, N, ld_x, ld_res, ld_out, ld_out_res, eps);
+    else
+      hipLaunchKernelGGL(rms_norm_f32_kernel<false>, grid, block, 0, s, (const float*)x,
+                         (const float*)weight, (const float*)residual, (float*)out,
+                         (float*)out_residual, N, ld_x, ld_res, ld_out, ld_out_res, eps);
+    return launch_status();
+  }
 #define DLB_LAUNCH_NORM(DT_, ADD_)                                                            \
   hipLaunchKernelGGL((rms_norm_kernel<DT_, ADD_>), grid, block, 0, s, (const unsigned short*)x, \
                      (const unsigned short*)weight, (const unsigned short*)residual,          \
@@ -319,18 +412,25 @@ extern "C" int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void
   if (num_tokens < 0 || Hq < 0 || Hk < 0 || D < 2) return DLB_ERR_BAD_ARG;
   if (num_tokens == 0 || Hq + Hk == 0) return DLB_OK;
   if (!q || !k || !cos || !sin || !q_out || !k_out) return DLB_ERR_BAD_ARG;
-  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
-  if (D % 16 != 0 || num_tokens > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
+  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16 && dtype != DLB_DTYPE_F32)
+    return DLB_ERR_UNSUPPORTED;
+  const int vec = dtype == DLB_DTYPE_F32 ? 4 : 8;  // elements per 16-byte vector
+  if (D % (2 * vec) != 0 || num_tokens > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
   const int64_t strides[] = {q_stride_tok,  q_stride_head,  k_stride_tok,  k_stride_head, qo_stride_tok,
                              qo_stride_head, ko_stride_tok, ko_stride_head, cs_stride_tok};
   for (int64_t sd : strides)
-    if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
+    if (sd % vec != 0) return DLB_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(k) || !aligned16(cos) || !aligned16(sin) || !aligned16(q_out) ||
       !aligned16(k_out))
     return DLB_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)num_tokens), block(256);
-  if (dtype == DLB_DTYPE_BF16)
+  if (dtype == DLB_DTYPE_F32)
+    hipLaunchKernelGGL(rotary_f32_kernel, grid, block, 0, s, (const float*)q, (const float*)k,
+                       (const float*)cos, (const float*)sin, (float*)q_out, (float*)k_out, Hq, Hk,
+                       D, q_stride_tok, q_stride_head, k_stride_tok, k_stride_head, qo_stride_tok,
+                       qo_stride_head, ko_stride_tok, ko_stride_head, cs_stride_tok);
+  else if (dtype == DLB_DTYPE_BF16)
     hipLaunchKernelGGL(rotary_kernel<DLB_DTYPE_BF16>, grid, block, 0, s, (const unsigned short*)q,
                        (const unsigned short*)k, (const unsigned short*)cos,
                        (const unsigned short*)sin, (unsigned short*)q_out, (unsigned short*)k_out,

@@ -324,15 +324,16 @@ int dlb_fill_kv_cache(const void* k_states, const void* v_states, void* k_cache,
 /* rms_norm: out = weight * round(x * rsqrt(mean(x^2) + eps)); with `residual` != NULL the
  * input is first replaced by round(x + residual), which is also written to out_residual.
  * Replaces rms_norm / add_rms_norm, kernels/rms_norm.py:8-133 and kernels/add_rms_norm.py:9-80.
- * x/out/residual/out_residual [M, N] with row strides, weight [N]; bf16/f16, N % 8 == 0,
- * N <= 16384. */
+ * x/out/residual/out_residual [M, N] with row strides, weight [N]; bf16/f16 (N % 8 == 0) or
+ * f32 (N % 4 == 0; nothing is rounded on the way), N <= 16384, 16-byte aligned rows. */
 int dlb_rms_norm(const void* x, const void* weight, const void* residual, void* out,
                  void* out_residual, int64_t M, int N, int64_t ld_x, int64_t ld_res,
                  int64_t ld_out, int64_t ld_out_res, float eps, int dtype, void* stream);
 
 /* apply_rotary_pos_emb: out = x * cos + rotate_half(x) * sin on q [T, Hq, D] and k [T, Hk, D],
  * cos/sin [T, D] (row stride cs_stride_tok); outputs may alias the inputs.
- * Replaces apply_rotary_pos_emb, kernels/apply_rotary_pos_emb.py:8-164.  bf16/f16, D % 16 == 0. */
+ * Replaces apply_rotary_pos_emb, kernels/apply_rotary_pos_emb.py:8-164.  bf16/f16 (D % 16 == 0)
+ * or f32 (D % 8 == 0); strides multiples of a 16-byte vector. */
 int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void* cos, const void* sin,
                              void* q_out, void* k_out, int64_t num_tokens, int Hq, int Hk, int D,
                              int64_t q_stride_tok, int64_t q_stride_head, int64_t k_stride_tok,

@@ -55,9 +55,12 @@ def test_fill_kv_cache_odd_head_dims_and_views(dev):
     assert torch.equal(kcd.cpu(), rk) and torch.equal(vcd.cpu(), rv)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("shape", [(4, 8), (3, 7, 4096), (64, 2048), (5, 11008), (2, 16384)])
+# test_rms_norm.py:33-35: bf16, fp16 and fp32 on a (4, 8) input
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(4, 8), (3, 7, 4096), (64, 2048), (5, 11008), (2, 16384), (6, 12)])
 def test_rms_norm(dev, dtype, shape):
+    if shape[-1] % 8 != 0 and dtype != torch.float32:
+        pytest.skip("16-bit rows are handled in 8-element vectors")
     from dlcompiler_amd.kernels.rms_norm import add_rms_norm, rms_norm
 
     g = torch.Generator().manual_seed(2)
@@ -69,6 +72,8 @@ def test_rms_norm(dev, dtype, shape):
     # the row sum is accumulated in a different order, which can flip the first of the two
     # roundings (normalise, then times weight) by one ulp -> allow two fp16 ulps
     tol = dict(rtol=2e-3, atol=1e-5) if dtype == torch.float16 else dict(rtol=1.6e-2, atol=1e-5)
+    if dtype == torch.float32:  # assert_close's default for fp32 (1.3e-6) plus the sum order
+        tol = dict(rtol=5e-6, atol=1e-6)
     torch.testing.assert_close(out, ref, **tol)
     res = torch.randn(shape, generator=g).to(dtype)
     rout, rres = od.rms_norm(x, w, 1e-6, residual=res)
@@ -80,8 +85,8 @@ def test_rms_norm(dev, dtype, shape):
     assert torch.equal(o3.cpu().reshape(shape), out2.cpu()) and torch.equal(r3.cpu().reshape(shape), res2.cpu())
 
 
-# test_apply_rotary.py:71-85: heads (8,8)/(8,4), feature dim 16, bf16/fp16, random positions
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+# test_apply_rotary.py:71-90: heads (8,8)/(8,4), feature dim 16, bf16/fp16/fp32, random positions
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("hq,hk,d", [(8, 8, 16), (8, 4, 16), (32, 8, 128), (5, 1, 64)])
 def test_apply_rotary(dev, dtype, hq, hk, d):
     from dlcompiler_amd.kernels.apply_rotary_pos_emb import apply_rotary_pos_emb
@@ -96,6 +101,8 @@ def test_apply_rotary(dev, dtype, hq, hk, d):
     rq, rk = od.apply_rotary_pos_emb(q.float(), k.float(), cos.float(), sin.float())
     qe, ke = apply_rotary_pos_emb(q.to(dev), k.to(dev), cos.to(dev), sin.to(dev))
     tol = dict(rtol=1e-5, atol=1e-3) if dtype == torch.float16 else dict(rtol=1.6e-2, atol=1e-5)
+    if dtype == torch.float32:  # products may be contracted into fused multiply-adds
+        tol = dict(rtol=1e-6, atol=1e-6)
     torch.testing.assert_close(qe.cpu().float(), rq, **tol)
     torch.testing.assert_close(ke.cpu().float(), rk, **tol)
     # and against the reference ground truth evaluated in the storage dtype
