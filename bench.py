@@ -69,6 +69,7 @@ class Timer:
 
 
 MIN_WARMUP = 10       # warm-up iterations before any timed region, whatever --warmup says
+MIN_WARMUP_S = 0.05   # ... and at least this much wall time of warm-up steps
 STAT_ITERS = 100      # iterations behind the median / p10 / p90 figures
 STAT_BATCHES = 20
 
@@ -87,13 +88,22 @@ def _time_steps(step, steps, warmup):
     ms_per_step: the K = `steps` timed steps are bracketed by one event before and one after on
     the launch stream, and nothing else is recorded inside the region (an event pair around every
     step costs about 10 us of host time and 7 us of GPU time per step -- a quarter of the shortest
-    workload).  At least MIN_WARMUP untimed steps run first.
+    workload).  At least MIN_WARMUP untimed steps and MIN_WARMUP_S seconds of them run first.
     stats: STAT_ITERS further iterations in STAT_BATCHES batches, one event pair per batch; the
     median / p10 / p90 are over the per-step times of the batches (batch time / batch size).  For
     a single-kernel workload a step is that kernel's launch, launch gaps included."""
-    for i in range(warmup if COUNTER_PASS else max(warmup, MIN_WARMUP)):
+    t0 = time.perf_counter()
+    n_warm = warmup if COUNTER_PASS else max(warmup, MIN_WARMUP)
+    for i in range(n_warm):
         step(i)
     torch.cuda.synchronize()
+    # a workload of a few microseconds per step has not brought the chip out of its idle clocks
+    # after ten steps: keep warming (untimed) until MIN_WARMUP_S of wall time have passed
+    while not COUNTER_PASS and time.perf_counter() - t0 < MIN_WARMUP_S and n_warm < 20000:
+        for i in range(10):
+            step(n_warm + i)
+        n_warm += 10
+        torch.cuda.synchronize()
     t_all = Timer()
     ev = t_all.start()
     for i in range(steps):
