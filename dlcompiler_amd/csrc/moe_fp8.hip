@@ -425,14 +425,20 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
     x[0] = *(const u32x4*)(base + (f0 ^ (hk << 6)));
     x[1] = *(const u32x4*)(base + (f0 ^ (hk << 6) ^ 32));
   };
+  // max(scale, floor) as ONE integer maximum on the bit patterns (positive floats order like
+  // their bits; a negative or zero scale becomes the floor): fmaxf costs a second instruction
+  // that quiets NaNs, and these sit in the main loop
+  auto floor_scale = [&](float v) -> float {
+    return __int_as_float(max(__float_as_int(v), __float_as_int(kScaleFloor)));
+  };
   // row 32 rt + j's activation scale sits in wave rt's strip of the chunk's slot
   const unsigned char* as_mine = sc_lds + j * 4;
   auto read_as = [&](int slot, int rt) -> float {
-    return fmaxf(*(const float*)(as_mine + slot * kScSlot + rt * kScWave), kScaleFloor);
+    return floor_scale(*(const float*)(as_mine + slot * kScSlot + rt * kScWave));
   };
   // (wave-uniform)
   auto read_ws = [&](int kc, int ct) -> float {
-    return fmaxf(ws_lds[wave][ct][kc], kScaleFloor);
+    return floor_scale(ws_lds[wave][ct][kc]);
   };
 
   f32x16 acc[NRT][2];  // [row tile][column tile]
