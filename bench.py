@@ -677,6 +677,81 @@ def wl_paged_prefill(dev, steps, warmup, cpu):
     return res
 
 
+def measure_box(dev):
+    """What this chip sustains, measured in this run: the matrix-instruction rate on random and on
+    all-zero operands (the clock under matrix load follows the power the operand data draws, so
+    the two differ by a third; the published peaks correspond to the all-zero case) and the rate
+    of a plain non-temporal stream.  Reported beside every roofline, never instead of it."""
+    from dlcompiler_amd import _lib
+
+    lib = _lib.load()
+    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
+    nbytes = lib.dlb_probe_mfma_operand_bytes(blocks)
+    sink = torch.zeros(512, dtype=torch.float32, device=dev)
+    stream = _lib.current_stream_ptr(dev)
+    g = _gen(99)
+    n16 = nbytes // 2
+    operands = {
+        "bf16_randn": torch.randn(n16, generator=g).bfloat16().to(dev),
+        "bf16_zeros": torch.zeros(n16, dtype=torch.bfloat16, device=dev),
+        "fp8_randn": torch.randn(nbytes, generator=g).to(torch.float8_e4m3fn).to(dev),
+        "fp8_zeros": torch.zeros(nbytes, dtype=torch.uint8, device=dev),
+    }
+    out = {}
+    for key, buf in operands.items():
+        fp8 = int(key.startswith("fp8"))
+        iters = 20000 if fp8 else 40000   # about 12 ms per launch on random operands
+
+        def launch():
+            _lib.check(lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), blocks, fp8,
+                                               iters, stream), "dlb_probe_mfma_rate")
+
+        for _ in range(3):
+            launch()
+        torch.cuda.synchronize()
+        t = Timer()
+        ev = t.start()
+        for _ in range(3):
+            launch()
+        t.stop(ev)
+        ms = t.mean_ms() / 3
+        flops = blocks * 8 * iters * 4 * (131072 if fp8 else 32768)
+        out[f"mfma_{key}_tflops"] = flops / ms / 1e9
+    x = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()   # 1 GiB
+    nb = x.numel() * 4
+
+    def read():
+        _lib.check(lib.dlb_probe_hbm_read(x.data_ptr(), sink.data_ptr(), nb, stream), "dlb_probe_hbm_read")
+
+    for _ in range(3):
+        read()
+    torch.cuda.synchronize()
+    t = Timer()
+    ev = t.start()
+    for _ in range(10):
+        read()
+    t.stop(ev)
+    out["hbm_read_gbs"] = nb / (t.mean_ms() / 10) / 1e6
+    out["note"] = ("measured in this run: back-to-back MFMAs (bf16 32x32x16 / fp8 32x32x64, two waves "
+                   "per SIMD on every CU, nothing else in the loop) on random-normal and on all-zero "
+                   "operands; a read-only non-temporal stream over 1 GiB")
+    del x
+    torch.cuda.empty_cache()
+    return out
+
+
+def _add_measured_ceiling(res, box):
+    """roofline.measured_peak / frac_of_measured: the same achieved figure against what the chip
+    sustained in this run on random operands (MFMA-bound) or in a read-only stream (HBM-bound)."""
+    rf = res["roofline"]
+    if rf["bound"] == "mfma":
+        peak = box["mfma_fp8_randn_tflops"] if rf["peak"] == PEAK_FP8_TFLOPS else box["mfma_bf16_randn_tflops"]
+    else:
+        peak = box["hbm_read_gbs"]
+    rf["measured_peak"] = peak
+    rf["frac_of_measured"] = rf["achieved"] / peak
+
+
 WORKLOADS = {
     "silu_and_mul": wl_silu,
     "moe_gating": wl_gating,
@@ -729,6 +804,13 @@ def main():
         torch.cuda.synchronize()
         del x, y
         torch.cuda.empty_cache()
+    box = None if args.counters else measure_box(dev)
+    if box is not None:
+        print("[bench] this chip, measured: MFMA bf16 %.0f TFLOP/s on random operands (%.0f on zeros), "
+              "fp8 %.0f (%.0f), read-only HBM stream %.0f GB/s" % (
+                  box["mfma_bf16_randn_tflops"], box["mfma_bf16_zeros_tflops"],
+                  box["mfma_fp8_randn_tflops"], box["mfma_fp8_zeros_tflops"], box["hbm_read_gbs"]),
+              file=sys.stderr, flush=True)
     names = list(WORKLOADS) if args.workload == "all" else [args.workload]
     primary = PRIMARY if args.workload == "all" else args.workload
     results = {}
@@ -737,6 +819,8 @@ def main():
         results[name] = WORKLOADS[name](dev, args.steps, args.warmup, not args.no_cpu)
         torch.cuda.synchronize()
         torch.cuda.empty_cache()
+        if box is not None:
+            _add_measured_ceiling(results[name], box)
         print(f"[bench] {name}: {results[name]['value']:.2f} {results[name]['unit']} "
               f"({results[name]['ms_per_step'] * 1e3:.1f} us/step, roofline "
               f"{results[name]['roofline']['frac'] * 100:.1f}%) in {time.perf_counter() - t0:.1f}s",
@@ -750,6 +834,7 @@ def main():
         "cpu_baseline": p.get("cpu_baseline"),
         "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
                  "cpu_model": _cpu_model()},
+        "box": box,
         "workloads": results,
     }
     print(json.dumps(line))

@@ -58,6 +58,9 @@ SIGNATURES = {
     "dlb_apply_rotary_pos_emb": (c_int, [c_void_p] * 6 + [c_int64, c_int, c_int, c_int]
                                  + [c_int64] * 9 + [c_int, c_void_p]),
     "dlb_moe_topk_sum": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_void_p]),
+    "dlb_probe_mfma_operand_bytes": (c_int64, [c_int]),
+    "dlb_probe_hbm_read": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "dlb_probe_mfma_rate": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None

@@ -341,6 +341,22 @@ int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void* cos, cons
                              int64_t ko_stride_tok, int64_t ko_stride_head, int64_t cs_stride_tok,
                              int dtype, void* stream);
 
+/* Measurement aid (no counterpart in the reference; used by bench.py, not by any operator):
+ * launches `blocks` workgroups of 512 threads that each issue `iters` rounds of four independent
+ * MFMAs per wave (bf16 32x32x16, or fp8 32x32x64 when fp8 != 0) on operand registers loaded once
+ * from `operands` -- no memory traffic, LDS or vector arithmetic in the loop.  Timed by the
+ * caller, it gives the matrix rate this chip sustains on that operand DATA (the clock under
+ * matrix load follows the power the data draws).  FLOPs = blocks * 8 waves * iters * 4 * (32768
+ * for bf16, 131072 for fp8).  operands: at least dlb_probe_mfma_operand_bytes(blocks) bytes,
+ * 16-byte aligned, any contents; sink: 2 KB the kernel practically never writes. */
+int64_t dlb_probe_mfma_operand_bytes(int blocks);
+/* Second measurement aid: reads `bytes` (a multiple of 16) from src with non-temporal 16-byte
+ * loads, eight in flight per lane, and discards them.  Timed by the caller it is the HBM rate a
+ * kernel with no arithmetic and no stores reaches on this chip. */
+int dlb_probe_hbm_read(const void* src, void* sink, int64_t bytes, void* stream);
+int dlb_probe_mfma_rate(const void* operands, int64_t operand_bytes, void* sink, int blocks,
+                        int fp8, int iters, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
