@@ -718,8 +718,11 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
           const int r = (tid_e >> 5) + 8 * i, pc = tid_e & 31;
           const int sid = sid_lds[64 * half + r];
           if (sid < p.numel && 8 * pc < ncols)
-            *(u32x4*)((unsigned short*)p.out + (int64_t)sid * p.N + nt * 256 + 8 * pc) =
-                *(const u32x4*)(x_lds + r * kPitch + 16 * pc);
+            // (non-temporal: the 100 MB of slot rows would otherwise push the weight lines that the
+            // expert's other row blocks are about to read out of L2)
+            __builtin_nontemporal_store(
+                *(const u32x4*)(x_lds + r * kPitch + 16 * pc),
+                (u32x4*)((unsigned short*)p.out + (int64_t)sid * p.N + nt * 256 + 8 * pc));
         }
         if (half + 1 < NRT / 2) __syncthreads();  // the second half reuses the staging rows
       }
