@@ -15,10 +15,7 @@
 //     from ds_read_b64_tr_b16, which hands lane l of a 16-lane group column l of a 4-row x
 //     16-column block (rows supplied by lanes 4j .. 4j+3), i.e. the transpose happens in the
 //     LDS read and V never passes through registers on its way in;
-//   * the exponent runs in base 2: Q is multiplied by scale * log2(e) once when it is loaded, and
-//     the score accumulators start at minus the running reference, so the MFMAs deliver the
-//     argument of exp2 and the softmax costs one maximum, one exponential and one addition per
-//     score;
+//   * the exponent runs in base 2 with the softmax scale folded into one FMA;
 //   * fully masked tiles are skipped per wave and only diagonal tiles pay for the mask; the
 //     heaviest query tiles are launched first.
 #include <type_traits>
@@ -66,10 +63,6 @@ struct Mma32<DLB_DTYPE_BF16> {
     f2 f = {a, b};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, b2));
   }
-  // both elements of a packed pair times c, rounded back to the element type
-  static __device__ __forceinline__ unsigned int scale2(unsigned int w, float c) {
-    return pack2(__uint_as_float(w << 16) * c, __uint_as_float(w & 0xffff0000u) * c);
-  }
 };
 template <>
 struct Mma32<DLB_DTYPE_F16> {
@@ -82,12 +75,6 @@ struct Mma32<DLB_DTYPE_F16> {
     typedef __attribute__((ext_vector_type(2))) _Float16 h2;
     f2 f = {a, b};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, h2));
-  }
-  static __device__ __forceinline__ unsigned int scale2(unsigned int w, float c) {
-    typedef __attribute__((ext_vector_type(2))) float f2;
-    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
-    const f2 f = __builtin_convertvector(__builtin_bit_cast(h2, w), f2);
-    return pack2(f[0] * c, f[1] * c);
   }
 };
 
@@ -171,9 +158,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   const unsigned short* kb = (const unsigned short*)p.k + (int64_t)kvh * p.k_sh;
   const unsigned short* vb = (const unsigned short*)p.v + (int64_t)kvh * p.v_sh;
 
-  // ---- Q^T as B operand: lane (n = query, k = dims 16*ks + 8*hh .. +8), kept in registers,
-  // multiplied once by scale * log2(e) (and rounded back to the element type) so that the score
-  // MFMAs deliver exponents of 2 directly
+  // ---- Q^T as B operand: lane (n = query, k = dims 16*ks + 8*hh .. +8), kept in registers
   const int qrow = q0 + 32 * wave + col;
   u32x4 qf[KS];
   {
@@ -183,8 +168,6 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     for (int ks = 0; ks < KS; ++ks) {
       qf[ks] = u32x4{0u, 0u, 0u, 0u};
       if (!RAGGED || 16 * ks + 8 * hh < p.dk) qf[ks] = *(const u32x4*)(qp + 16 * ks);
-#pragma unroll
-      for (int w = 0; w < 4; ++w) qf[ks][w] = Mma32<DT>::scale2(qf[ks][w], p.scale_log2e);
     }
   }
 
@@ -315,15 +298,10 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   // lazily: the accumulators are rescaled only when a row maximum exceeds it by more than
   // kRescaleGap, so between rescales probabilities stay below 2^kRescaleGap -- exact in the
   // end (the same factor cancels in O / l), and it removes the per-tile rescale of O.
-  // The reference is not subtracted by vector instructions: the score accumulators START at
-  // -m_run (neg_ref, the C operand of the first k-step), so the MFMAs deliver s - m_run and the
-  // exponential is the only per-score instruction besides the maximum and the sum.
   constexpr float kRescaleGap = 8.0f;
-  float m_run = -__builtin_inff();  // -inf: no visible key seen yet (the accumulators then start at 0)
+  float m_run = -__builtin_inff();
   float l_run = 0.0f;  // this lane half's share of the denominator
-  f32x16 neg_ref;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) neg_ref[i] = 0.0f;
+  const float cs = p.scale_log2e;
 
   // byte offsets of this lane's transposing V reads inside a tile, one per 32-dim block
   int v_off[MT];
@@ -353,6 +331,10 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
     // k-step outer, key tile inner: two independent accumulator chains, and the K fragments
     // are fetched from LDS two k-steps ahead of the MFMAs that consume them
     f32x16 s[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[nt][i] = 0.0f;
     // MFMA-dense phase: let this wave's issue win over the other wave of the SIMD, whose
     // softmax arithmetic then fills the gaps while the matrix pipe is busy
     __builtin_amdgcn_s_setprio(1);
@@ -374,15 +356,14 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         if (kstep + kAhead < KS) ldk(kstep + kAhead, ka[(kstep + kAhead) % (kAhead + 1)]);
         if (COPY) issue_copy(kstep);
         __builtin_amdgcn_sched_barrier(0);  // keep the fetch ahead of the MFMAs (it would be sunk)
-        s[0] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][0], qf[kstep], kstep == 0 ? neg_ref : s[0]);
-        s[1] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][1], qf[kstep], kstep == 0 ? neg_ref : s[1]);
+        s[0] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][0], qf[kstep], s[0]);
+        s[1] = Mma32<DT>::run(ka[kstep % (kAhead + 1)][1], qf[kstep], s[1]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
 
     __builtin_amdgcn_s_setprio(0);
-    // ---- causal mask and tile maximum of the scores, which arrive relative to the reference
-    const float m_ref = (m_run == -__builtin_inff()) ? 0.0f : m_run;  // what neg_ref holds, negated
+    // ---- causal mask and tile maximum of the raw scores (scale > 0 commutes with max)
     float mpart[2] = {-__builtin_inff(), -__builtin_inff()};  // two independent chains
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
@@ -391,10 +372,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         if (MASK) {
           const int key = t0 + 32 * nt + 8 * (i >> 2) + 4 * hh + (i & 3);
           float x = s[nt][i];
-          if (softcap > 0.0f) {  // cap * tanh(score * scale / cap), all in log2 units
-            const float cap2 = softcap * 1.4426950408889634f;
-            x = tanhf((x + m_ref) / cap2) * cap2 - m_ref;
-          }
+          if (softcap > 0.0f)  // cap * tanh(x * scale / cap), kept in raw-score units
+            x = tanhf(x * (p.sm_scale / softcap)) * (softcap / p.sm_scale);
           bool vis = key <= qpos;
           if (window > 0) vis = vis && (key >= qpos - window);
           s[nt][i] = vis ? x : -__builtin_inff();
@@ -402,36 +381,29 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
         mpart[nt] = fmaxf(mpart[nt], s[nt][i]);
       }
     }
-    const float mloc = max_xor32(fmaxf(mpart[0], mpart[1]));  // relative to the reference
-    const bool unset = m_run == -__builtin_inff();
-    // the reference moves when a row maximum exceeds it by more than the gap, and is set by the
-    // first tile that shows the row a visible key (whatever its sign: it may lie far below 0)
-    if (__any(mloc > kRescaleGap || (unset && mloc > -__builtin_inff()))) {
-      // rows still without a visible key stay unset; rows that are set only move up
-      const float delta = unset ? mloc : fmaxf(mloc, 0.0f);  // -inf only for rows that stay unset
-      const bool stay = unset && mloc == -__builtin_inff();
-      const float d = stay ? 0.0f : delta;
-      const float alpha = unset ? 1.0f : __builtin_amdgcn_exp2f(-d);  // o and l are 0 while unset
-      if (!stay) m_run = m_ref + d;
+    // (the scale is applied here, to fp32 scores, as the reference does: folded into Q -- which
+    // would save the multiply-add below -- it is rounded to the element type, an error that
+    // grows with the score and reaches several percent of the probabilities at |score| ~ 100)
+    const float mloc = max_xor32(fmaxf(mpart[0], mpart[1])) * cs;
+    if (__any(mloc > m_run + kRescaleGap)) {
+      const float m_new = fmaxf(m_run, mloc);  // finite from tile 0 on (key 0 is visible)
+      // (a fully masked row under a sliding window keeps m_new = -inf: leave it untouched)
+      const float alpha = (MASK && PAGED && m_new == -__builtin_inff()) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
       l_run *= alpha;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[mt][i] *= alpha;
-      const float nr = stay ? 0.0f : -m_run;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) neg_ref[i] = nr;
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[nt][i] -= d;
     }
+    // a row whose keys so far were all masked (sliding window) still has m_run = -inf
+    const float m_ref = (MASK && PAGED && m_run == -__builtin_inff()) ? 0.0f : m_run;
     float psum = 0.0f;
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float e = __builtin_amdgcn_exp2f(s[nt][i]);
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][i], cs, -m_ref));
         s[nt][i] = e;
         psum += e;
       }
@@ -537,7 +509,7 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk,
     if (sd % 8 != 0) return DLB_ERR_UNSUPPORTED;
   if (p.o_st % 4 != 0 || p.o_sh % 4 != 0) return DLB_ERR_UNSUPPORTED;
   if (B > 65535) return DLB_ERR_UNSUPPORTED;
-  if (!(sm_scale > 0.0f)) return DLB_ERR_BAD_ARG;
+  if (!(sm_scale > 0.0f)) return DLB_ERR_BAD_ARG;  // the tile maximum is taken before scaling
 
   p.Hq = Hq;
   p.Hkv = Hkv;

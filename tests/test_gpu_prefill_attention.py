@@ -139,3 +139,30 @@ def test_config3_full(dev):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_head_sizes(dev, d, dtype):
     _run(dev, [1, 33, 64, 129, 700], 8, 2, d, dtype, gap=2)
+
+
+# the exponent reference of a row is set by its first tile and only moves up by steps larger
+# than 8: scores far below zero, far above it, and a late key that dwarfs everything before it
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_score_ranges(dev, dtype):
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    L, hq, hkv, d = 300, 4, 2, 128
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn((L, hq, d), generator=g)
+    k = torch.randn((L, hkv, d), generator=g)
+    v = torch.randn((L, hkv, d), generator=g).to(dtype)
+    start, seqlen = torch.tensor([0], dtype=torch.int32), torch.tensor([L], dtype=torch.int32)
+    cases = {
+        "large negative scores": (q * 6, -q[:, :hkv].abs().mean(0, keepdim=True).expand(L, hkv, d) * 6 + k * 0.1),
+        "large positive scores": (q.abs() * 4, k.abs() * 4),
+        "late dominant key": (q, torch.cat([k[:200] * 0.05, k[200:201] * 0 + q[250, :hkv] * 3, k[201:] * 0.05])),
+    }
+    for name, (qq, kk) in cases.items():
+        qq, kk = qq.to(dtype), kk.to(dtype)
+        ref = oa.prefill_attention(qq, kk, v, start, seqlen)
+        o = torch.empty((L, hq, d), dtype=dtype, device=dev)
+        context_attention_fwd(qq.to(dev), kk.to(dev), v.to(dev), o, start.to(dev), seqlen.to(dev), L)
+        out = o.cpu().float()
+        assert torch.isfinite(out).all(), name
+        torch.testing.assert_close(out, ref.float(), rtol=2e-2, atol=2e-2, msg=lambda m: f"{name}: {m}")
