@@ -89,6 +89,54 @@ def test_decode_sweep(dev, seed):
     _close(o.cpu(), oa.paged_decode(q, kc, vc, table, kl, window=window, softcap=softcap))
 
 
+# head sizes that are any multiple of 8 (key and value size drawn independently), all three paths
+@pytest.mark.parametrize("seed", range(16))
+def test_head_size_sweep(dev, seed):
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    rng = random.Random(300 + seed)
+    d = 8 * rng.randint(1, 16)
+    dv = rng.choice([d, 8 * rng.randint(1, 16)])
+    hkv = rng.choice([1, 2])
+    hq = hkv * rng.choice([1, 4])
+    dtype = rng.choice([torch.bfloat16, torch.float16])
+    gen = torch.Generator().manual_seed(3000 + seed)
+    nseq = rng.randint(1, 3)
+    lens = [rng.choice(_LENS) for _ in range(nseq)]
+    T = sum(lens)
+    start = torch.tensor([sum(lens[:i]) for i in range(nseq)], dtype=torch.int32)
+    sl = torch.tensor(lens, dtype=torch.int32)
+    q = torch.randn((T, hq, d), generator=gen).to(dtype)
+
+    # packed prefill (one head size for q, k and v)
+    k = torch.randn((T, hkv, d), generator=gen).to(dtype)
+    v = torch.randn((T, hkv, d), generator=gen).to(dtype)
+    o = torch.zeros_like(q, device=dev)
+    context_attention_fwd(q.to(dev), k.to(dev), v.to(dev), o, start.to(dev), sl.to(dev), max(lens))
+    _close(o.cpu(), oa.prefill_attention(q, k, v, start, sl))
+
+    # paged prefill after a history and paged decode, value size dv
+    page = rng.choice([16, 32, 64])
+    hist = [rng.choice([0, 17, 100]) for _ in range(nseq)]
+    full = [a + b for a, b in zip(lens, hist)]
+    ks = [torch.randn((n, hkv, d), generator=gen).to(dtype) for n in full]
+    vs = [torch.randn((n, hkv, dv), generator=gen).to(dtype) for n in full]
+    kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=seed, dtype=dtype)
+    ql, kl = torch.tensor(lens), torch.tensor(full)
+    if T != nseq:
+        o2 = torch.zeros((T, hq, dv), dtype=dtype, device=dev)
+        paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o2, table.to(dev), start.to(dev),
+                            ql.to(dev), kl.to(dev), max(lens))
+        _close(o2.cpu(), oa.paged_prefill(q, kc, vc, table, start.long(), ql, kl))
+    qd = torch.randn((nseq, hq, d), generator=gen).to(dtype)
+    o3 = torch.zeros((nseq, hq, dv), dtype=dtype, device=dev)
+    paged_attention_fwd(qd.to(dev), kc.to(dev), vc.to(dev), o3, table.to(dev),
+                        torch.arange(nseq, device=dev), torch.ones(nseq, dtype=torch.int64, device=dev),
+                        kl.to(dev), 1)
+    _close(o3.cpu(), oa.paged_decode(qd, kc, vc, table, kl))
+
+
 def test_config_size_attention_repeats_bit_identically(dev):
     """Config-size prefill and paged decode, repeated: both kernels copy K/V into LDS with
     hand-issued loads and explicit waits; a missing wait would show as run-to-run differences."""
