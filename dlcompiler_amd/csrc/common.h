@@ -47,8 +47,12 @@ struct Elem<DLB_DTYPE_BF16> {
   static __device__ __forceinline__ float hi(unsigned int w) {
     return __uint_as_float(w & 0xffff0000u);
   }
+  // two floats -> two bf16 in one word: v_cvt_pk_bf16_f32 (round to nearest even, NaN quiet)
   static __device__ __forceinline__ unsigned int pack(float a, float b) {
-    return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+    const f2 f = {a, b};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, b2));
   }
   static __device__ __forceinline__ float load1(const void* p, int64_t i) {
     return bf16_bits_to_f32(((const unsigned short*)p)[i]);
@@ -62,7 +66,10 @@ struct Elem<DLB_DTYPE_F16> {
   static __device__ __forceinline__ float lo(unsigned int w) { return f16_bits_to_f32(w & 0xffffu); }
   static __device__ __forceinline__ float hi(unsigned int w) { return f16_bits_to_f32(w >> 16); }
   static __device__ __forceinline__ unsigned int pack(float a, float b) {
-    return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    const f2 f = {a, b};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, h2));
   }
   static __device__ __forceinline__ float load1(const void* p, int64_t i) {
     return f16_bits_to_f32(((const unsigned short*)p)[i]);
