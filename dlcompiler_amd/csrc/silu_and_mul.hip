@@ -5,9 +5,10 @@
 // gate / (1 + exp(-gate)) * up, one rounding to the output type at the store.
 //
 // The op is a pure HBM stream (3 bytes moved per output byte), so the kernel is built around
-// 128-bit accesses: each lane owns 16-byte vectors of gate and up, UNROLL of them in flight
-// before the first use, and the grid is flattened over M * N / VEC so that a row length that
-// is not a multiple of the block (N = 11008 -> 1376 vectors) leaves no idle lanes.
+// 128-bit accesses: each lane owns 16-byte vectors of gate and up (UNROLL pairs, all requested
+// before the first use; one pair per lane and many resident waves turned out fastest), and the
+// grid is flattened over M * N / VEC so that a row length that is not a multiple of the block
+// (N = 11008 -> 1376 vectors) leaves no idle lanes.
 #include "common.h"
 
 namespace dlb {
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_scalar(const void* __restric
 template <int DT>
 int launch_16bit(const void* x, void* out, int64_t M, int64_t N, int64_t ldx, int64_t ldo,
                  hipStream_t s) {
-  constexpr int VEC = 8, UNROLL = 4;
+  constexpr int VEC = 8, UNROLL = 1;  // measured: 1 -> 85 us, 2 -> 86.5, 4 -> 91.5, 8 -> 98 at [8192, 2 x 11008]
   const int64_t total_vec = M * (N / VEC);
   const bool vec_ok = (N % VEC == 0) && (ldx % VEC == 0) && (ldo % VEC == 0) && aligned16(x) &&
                       aligned16(out) && total_vec < (int64_t)0xffffffffu - 256 * UNROLL &&
