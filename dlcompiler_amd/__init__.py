@@ -4,7 +4,8 @@ Module layout mirrors ``dlblas.kernels`` for the operators that are implemented:
 
 * ``dlcompiler_amd.kernels.activation.silu_and_mul``
 * ``dlcompiler_amd.kernels.prefill_attention.context_attention_fwd``
-* ``dlcompiler_amd.kernels.paged_attention.paged_attention_fwd`` (decode branch)
+* ``dlcompiler_amd.kernels.paged_attention.paged_attention_fwd`` (decode and prefill-with-history
+  branches, sliding window, logit soft-capping)
 * ``dlcompiler_amd.kernels.fused_moe.fused_moe`` / ``get_start_end`` and the fp8 variant
   ``fused_moe_fp8`` with ``per_token_group_quant_fp8`` / ``shuffle_moe_weight``
 * ``dlcompiler_amd.kernels.moe_gating.moe_topk_softmax`` / ``moe_align_block_size`` /
