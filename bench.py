@@ -677,6 +677,33 @@ def wl_paged_prefill(dev, steps, warmup, cpu):
     return res
 
 
+_probe_lib = None
+
+
+def load_probe_lib():
+    """ctypes binding of ``libdlblas_bench_probe.so`` (``dlcompiler_amd/csrc/bench/bench_probe.h``):
+    the two measurement kernels behind ``box``; a library of its own, built with the operators'."""
+    global _probe_lib
+    if _probe_lib is None:
+        import ctypes
+        from ctypes import c_int, c_int64, c_void_p
+
+        from dlcompiler_amd.build import PROBE_LIB_PATH
+
+        if not PROBE_LIB_PATH.exists():
+            raise ImportError(f"{PROBE_LIB_PATH} not found: build it with `python -m dlcompiler_amd.build`")
+        lib = ctypes.CDLL(str(PROBE_LIB_PATH))
+        lib.dlb_probe_mfma_operand_bytes.restype = c_int64
+        lib.dlb_probe_mfma_operand_bytes.argtypes = [c_int]
+        lib.dlb_probe_mfma_rate.restype = c_int
+        lib.dlb_probe_mfma_rate.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int,
+                                            c_void_p]
+        lib.dlb_probe_hbm_read.restype = c_int
+        lib.dlb_probe_hbm_read.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p]
+        _probe_lib = lib
+    return _probe_lib
+
+
 def measure_box(dev):
     """What this chip sustains, measured in this run: the matrix-instruction rate on random and on
     all-zero operands (the clock under matrix load follows the power the operand data draws, so
@@ -684,10 +711,11 @@ def measure_box(dev):
     of a plain non-temporal stream.  Reported beside every roofline, never instead of it."""
     from dlcompiler_amd import _lib
 
-    lib = _lib.load()
+    lib = load_probe_lib()
     blocks = torch.cuda.get_device_properties(dev).multi_processor_count
     nbytes = lib.dlb_probe_mfma_operand_bytes(blocks)
     sink = torch.zeros(512, dtype=torch.float32, device=dev)
+    sink_bytes = sink.numel() * 4
     stream = _lib.current_stream_ptr(dev)
     g = _gen(99)
     n16 = nbytes // 2
@@ -703,8 +731,8 @@ def measure_box(dev):
         iters = 20000 if fp8 else 40000   # about 12 ms per launch on random operands
 
         def launch():
-            _lib.check(lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), blocks, fp8,
-                                               iters, stream), "dlb_probe_mfma_rate")
+            _lib.check(lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sink_bytes,
+                                               blocks, fp8, iters, stream), "dlb_probe_mfma_rate")
 
         for _ in range(3):
             launch()
@@ -721,7 +749,8 @@ def measure_box(dev):
     nb = x.numel() * 4
 
     def read():
-        _lib.check(lib.dlb_probe_hbm_read(x.data_ptr(), sink.data_ptr(), nb, stream), "dlb_probe_hbm_read")
+        _lib.check(lib.dlb_probe_hbm_read(x.data_ptr(), sink.data_ptr(), sink_bytes, nb, stream),
+                   "dlb_probe_hbm_read")
 
     for _ in range(3):
         read()

@@ -14,6 +14,7 @@ _PKG_DIR = Path(__file__).resolve().parent
 DEFAULT_LIB_PATH = _PKG_DIR / "lib" / "libdlblas_hip.so"
 
 DLB_OK = 0
+ABI_VERSION = 3  # DLB_ABI_VERSION of include/dlblas_hip.h this binding was written against
 DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 
 # name -> (restype, argtypes); must list every symbol include/dlblas_hip.h declares
@@ -37,11 +38,11 @@ SIGNATURES = {
                                                c_int64, c_void_p, c_void_p, c_void_p, c_size_t,
                                                c_void_p]),
     "dlb_paged_decode_ws_bytes": (c_size_t, [c_int] * 6),
-    "dlb_paged_decode_attn": (c_int, [c_void_p] * 6 + [c_int] * 7 + [c_int64] * 11
+    "dlb_paged_decode_attn": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_int64] * 11
                               + [c_float, c_int, c_float, c_int, c_void_p, c_size_t, c_void_p]),
-    "dlb_prefill_attn_varlen": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 8
+    "dlb_prefill_attn_varlen": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_int64] * 8
                                 + [c_float, c_int, c_void_p]),
-    "dlb_paged_prefill_attn": (c_int, [c_void_p] * 8 + [c_int] * 8 + [c_int64] * 11
+    "dlb_paged_prefill_attn": (c_int, [c_void_p] * 8 + [c_int] * 9 + [c_int64] * 11
                                + [c_float, c_int, c_float, c_int, c_void_p]),
     "dlb_per_token_group_quant_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                               c_int64, c_int64, c_int64, c_int, c_void_p]),
@@ -51,16 +52,13 @@ SIGNATURES = {
     "dlb_moe_gemm_16bit_gate_up": (c_int, [c_void_p] * 4 + [c_int] * 10 + [c_void_p, c_int, c_void_p]),
     "dlb_moe_gemm_16bit_down": (c_int, [c_void_p] * 4 + [c_int, c_void_p] + [c_int] * 9
                                 + [c_void_p, c_int, c_void_p]),
-    "dlb_fill_kv_cache": (c_int, [c_void_p] * 8 + [c_int64] + [c_int] * 7 + [c_int64] * 11
+    "dlb_fill_kv_cache": (c_int, [c_void_p] * 8 + [c_int, c_int64] + [c_int] * 7 + [c_int64] * 11
                           + [c_void_p]),
     "dlb_rms_norm": (c_int, [c_void_p] * 5 + [c_int64, c_int] + [c_int64] * 4
                      + [c_float, c_int, c_void_p]),
     "dlb_apply_rotary_pos_emb": (c_int, [c_void_p] * 6 + [c_int64, c_int, c_int, c_int]
                                  + [c_int64] * 9 + [c_int, c_void_p]),
     "dlb_moe_topk_sum": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_int, c_void_p]),
-    "dlb_probe_mfma_operand_bytes": (c_int64, [c_int]),
-    "dlb_probe_hbm_read": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
-    "dlb_probe_mfma_rate": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None
@@ -89,6 +87,9 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError if the symbol is missing
         fn.restype = restype
         fn.argtypes = argtypes
+    if lib.dlb_version() != ABI_VERSION:
+        raise ImportError(f"{path} has ABI version {lib.dlb_version()}, this binding needs "
+                          f"{ABI_VERSION}: rebuild it with `python -m dlcompiler_amd.build`")
     _lib = lib
     return lib
 
@@ -97,6 +98,23 @@ def check(status: int, what: str) -> None:
     if status != DLB_OK:
         msg = load().dlb_status_string(status).decode()
         raise DlblasHipError(f"{what}: {msg} (status {status})")
+
+
+def index_arrays(*tensors):
+    """Prepare index tensors (block tables, lengths, start offsets) for an entry point with an
+    ``index64_mask`` argument: int32 and int64 tensors pass as they are (the kernels read either
+    width), any other integer type is converted to int32.  Returns the tensors (keep them
+    referenced until the launch is enqueued) and the mask whose bit i is set when tensor i is int64."""
+    import torch
+
+    out, mask = [], 0
+    for i, t in enumerate(tensors):
+        if t.dtype == torch.int64:
+            mask |= 1 << i
+        elif t.dtype != torch.int32:
+            t = t.to(torch.int32)
+        out.append(t)
+    return out, mask
 
 
 def torch_dtype_code(dtype) -> int:

@@ -26,6 +26,9 @@ CSRC_DIR = PKG_DIR / "csrc"
 LIB_DIR = PKG_DIR / "lib"
 OBJ_DIR = LIB_DIR / "obj"
 LIB_PATH = LIB_DIR / "libdlblas_hip.so"
+# measurement kernels that bench.py times; a library of their own, not part of the operator ABI
+PROBE_SRC = CSRC_DIR / "bench" / "probe.hip"
+PROBE_LIB_PATH = LIB_DIR / "libdlblas_bench_probe.so"
 INCLUDE_DIR = PKG_DIR.parent / "include"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -89,14 +92,24 @@ def parse_resource_remarks(stderr: str) -> dict[str, dict[str, int]]:
     return kernels
 
 
-def check_hand_scheduled(kernels: dict[str, dict[str, int]]) -> list[str]:
-    """Names (with the offending figures) of hand-scheduled kernels that use scratch or spill."""
+def check_hand_scheduled(kernels: dict[str, dict[str, int]], source_text: str = "") -> list[str]:
+    """Names (with the offending figures) of hand-scheduled kernels that use scratch or spill.
+
+    The check fails closed: a source that defines a hand-scheduled kernel (its tag appears in
+    ``source_text``) must yield at least one parsed report for it, and every such report must
+    carry both figures -- a compiler that prints the remarks differently, or not at all, stops
+    the build instead of passing it."""
     bad = []
+    for tag in HAND_SCHEDULED:
+        if tag in source_text and not any(tag in name for name in kernels):
+            bad.append(f"{tag}: defined in the source but no resource report was parsed for it")
     for name, r in kernels.items():
         if any(tag in name for tag in HAND_SCHEDULED):
-            if r.get("scratch_bytes", 0) or r.get("vgpr_spills", 0):
-                bad.append(f"{name}: scratch {r.get('scratch_bytes', 0)} B/lane, "
-                           f"{r.get('vgpr_spills', 0)} spilled VGPRs")
+            if "scratch_bytes" not in r or "vgpr_spills" not in r:
+                bad.append(f"{name}: resource report lacks the scratch or spill figure")
+            elif r["scratch_bytes"] or r["vgpr_spills"]:
+                bad.append(f"{name}: scratch {r['scratch_bytes']} B/lane, "
+                           f"{r['vgpr_spills']} spilled VGPRs")
     return bad
 
 
@@ -120,7 +133,7 @@ def _compile_one(src: Path, obj: Path, verbose: bool) -> None:
     kernels = parse_resource_remarks(proc.stderr)
     report = obj.with_suffix(".resources.json")
     report.write_text(json.dumps(kernels, indent=1, sort_keys=True))
-    bad = check_hand_scheduled(kernels)
+    bad = check_hand_scheduled(kernels, src.read_text())
     if bad:
         obj.unlink(missing_ok=True)
         raise RuntimeError(f"{src.name}: hand-scheduled kernels must not spill or use scratch:\n  "
@@ -150,7 +163,20 @@ def build_library(force: bool = False, verbose: bool = False, jobs: int | None =
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"link failed:\n{proc.stderr}")
+    build_probe_library(force)
     return LIB_PATH
+
+
+def build_probe_library(force: bool = False) -> Path:
+    """Build ``libdlblas_bench_probe.so`` (the measurement kernels bench.py times)."""
+    deps = [PROBE_SRC, *PROBE_SRC.parent.glob("*.h"), *_headers()]
+    if force or _stale(PROBE_LIB_PATH, deps):
+        cmd = [HIPCC, *[f for f in DEVICE_FLAGS if not f.startswith("-Rpass")], f"-I{INCLUDE_DIR}",
+               "-shared", str(PROBE_SRC), "-o", str(PROBE_LIB_PATH)]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {PROBE_SRC.name}:\n{proc.stderr}")
+    return PROBE_LIB_PATH
 
 
 def kernel_resources() -> dict[str, dict[str, int]]:

@@ -7,7 +7,8 @@
 // Every wave cycles through four operand pairs read once from `operands` (so the registers hold
 // the caller's data, whatever its entropy) and issues `iters` rounds of four independent MFMAs;
 // no memory traffic, LDS or vector arithmetic inside the loop.
-#include "common.h"
+#include "../common.h"
+#include "bench_probe.h"
 
 namespace dlb {
 namespace {
@@ -77,9 +78,11 @@ __global__ __launch_bounds__(256) void hbm_read_kernel(const u32x4* __restrict__
 }  // namespace
 }  // namespace dlb
 
-extern "C" int dlb_probe_hbm_read(const void* src, void* sink, int64_t bytes, void* stream) {
+extern "C" int dlb_probe_hbm_read(const void* src, void* sink, int64_t sink_bytes, int64_t bytes,
+                                  void* stream) {
   using namespace dlb;
   if (bytes < 0 || !src || !sink) return DLB_ERR_BAD_ARG;
+  if (sink_bytes < DLB_PROBE_SINK_BYTES) return DLB_ERR_WORKSPACE;
   if (bytes == 0) return DLB_OK;
   if (bytes % 16 != 0 || !aligned16(src)) return DLB_ERR_UNSUPPORTED;
   const uint64_t nvec = (uint64_t)bytes / 16;
@@ -96,9 +99,11 @@ extern "C" int64_t dlb_probe_mfma_operand_bytes(int blocks) {
 }
 
 extern "C" int dlb_probe_mfma_rate(const void* operands, int64_t operand_bytes, void* sink,
-                                   int blocks, int fp8, int iters, void* stream) {
+                                   int64_t sink_bytes, int blocks, int fp8, int iters,
+                                   void* stream) {
   using namespace dlb;
   if (blocks < 1 || iters < 0 || !operands || !sink) return DLB_ERR_BAD_ARG;
+  if (sink_bytes < DLB_PROBE_SINK_BYTES) return DLB_ERR_WORKSPACE;
   if (operand_bytes < dlb_probe_mfma_operand_bytes(blocks)) return DLB_ERR_WORKSPACE;
   if (!aligned16(operands)) return DLB_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;

@@ -1,7 +1,7 @@
 // Version and status helpers of the C ABI.
 #include "common.h"
 
-extern "C" int dlb_version(void) { return 1; }
+extern "C" int dlb_version(void) { return DLB_ABI_VERSION; }
 
 extern "C" const char* dlb_status_string(int status) {
   switch (status) {

@@ -224,6 +224,18 @@ __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) {
   return (a + b - 1) / b;
 }
 
+// Index arrays (sequence lengths, start offsets, block tables) arrive as int32 or as int64, as the
+// caller's framework holds them; element i is read as the 32-bit word i << sh (sh = 1: the low
+// half of a little-endian int64 -- the values are token counts and page numbers below 2^31).
+struct IdxArray {
+  const int32_t* p;
+  int sh;
+  __device__ __forceinline__ int operator[](int64_t i) const { return p[i << sh]; }
+};
+inline IdxArray idx_array(const void* p, int index64_mask, int bit) {
+  return IdxArray{(const int32_t*)p, (index64_mask >> bit) & 1};
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // tokens per workgroup of the fused router + chunk-histogram kernel = tokens per alignment chunk

@@ -22,10 +22,10 @@ struct FillParams {
   const unsigned char* vs;
   unsigned char* kc;
   unsigned char* vc;
-  const int32_t* q_start;
-  const int32_t* q_len;
-  const int32_t* kv_len;
-  const int32_t* block_table;
+  IdxArray q_start;
+  IdxArray q_len;
+  IdxArray kv_len;
+  IdxArray block_table;
   int64_t ks_tok, ks_head, vs_tok, vs_head;              // bytes
   int64_t kc_page, kc_slot, kc_head, vc_page, vc_slot, vc_head;  // bytes
   int64_t bt_stride;
@@ -296,9 +296,10 @@ inline bool mult16(int64_t v) { return (v & 15) == 0; }
 }  // namespace dlb
 
 extern "C" int dlb_fill_kv_cache(const void* k_states, const void* v_states, void* k_cache,
-                                 void* v_cache, const int32_t* q_start_loc,
-                                 const int32_t* q_seq_len, const int32_t* kv_seq_len,
-                                 const int32_t* block_table, int64_t num_tokens, int batch,
+                                 void* v_cache, const void* q_start_loc,
+                                 const void* q_seq_len, const void* kv_seq_len,
+                                 const void* block_table, int index64_mask, int64_t num_tokens,
+                                 int batch,
                                  int heads, int head_dim, int head_dim_v, int page, int max_blocks,
                                  int elem_size, int64_t ks_stride_tok, int64_t ks_stride_head,
                                  int64_t vs_stride_tok, int64_t vs_stride_head,
@@ -321,10 +322,11 @@ extern "C" int dlb_fill_kv_cache(const void* k_states, const void* v_states, voi
   p.vs = (const unsigned char*)v_states;
   p.kc = (unsigned char*)k_cache;
   p.vc = (unsigned char*)v_cache;
-  p.q_start = q_start_loc;
-  p.q_len = q_seq_len;
-  p.kv_len = kv_seq_len;
-  p.block_table = block_table;
+  if (index64_mask & ~15) return DLB_ERR_BAD_ARG;
+  p.q_start = idx_array(q_start_loc, index64_mask, 0);
+  p.q_len = idx_array(q_seq_len, index64_mask, 1);
+  p.kv_len = idx_array(kv_seq_len, index64_mask, 2);
+  p.block_table = idx_array(block_table, index64_mask, 3);
   p.ks_tok = ks_stride_tok * es;
   p.ks_head = ks_stride_head * es;
   p.vs_tok = vs_stride_tok * es;

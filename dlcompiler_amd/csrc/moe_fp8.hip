@@ -33,6 +33,17 @@ namespace {
 
 constexpr float kFp8Max = 448.0f;
 constexpr float kQuantEps = 1e-10f;
+// K chunks of 128 bytes whose block scales the fp8 grouped GEMM parks in LDS: reduction lengths
+// up to 128 * 128 = 16384 (checked on the host before the launch)
+constexpr int kMoeMaxKChunks = 128;
+// Floors of the scales inside the fp8 GEMM.  The accumulators are kept relative to the scale of
+// the current K chunk (multiplied by s(k) / s(k + 1) between chunks), so |sum| / s(k) must stay
+// inside fp32: with the activation scale floored just below the smallest value the quantiser
+// itself produces (1e-10 / 448 = 2.2e-13, the scale of an all-zero group) and the weight block
+// scale floored at 1e-12 (a block whose values are below 4.5e-10), a row may mix empty groups,
+// empty weight blocks and groups of any realistic magnitude without leaving the fp32 range.
+constexpr float kActScaleFloor = 1e-13f;
+constexpr float kWScaleFloor = 1e-12f;
 
 __device__ __forceinline__ unsigned int pack4_fp8(float a, float b, float c, float d) {
   // v_cvt_pk_fp8_f32 rounds to nearest even; values beyond +-464 would become NaN, so clamp.
@@ -248,7 +259,8 @@ __device__ __forceinline__ bool find_tile(const MoeGemmParams& p, int lane, Tile
 // epilogue multiplies by the last s.  One multiply per accumulator and chunk, as many vector
 // operations as acc += P * s would take, but no separate product tile: 128 accumulators, two
 // chunks of weights and two fragment buffers fit the 256 registers of a wave at two waves per
-// SIMD.  (Scales are floored at 1e-30 so that a zero scale cannot divide.)
+// SIMD.  (Scales are floored -- kActScaleFloor, kWScaleFloor -- so that a zero scale cannot
+// divide and the ratio of two neighbouring chunks cannot push an accumulator out of fp32.)
 //
 // Data movement:
 //   * weights: global -> operand registers with plain loads, in units of (chunk half, both
@@ -271,10 +283,9 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
   constexpr int NX = 3;                 // activation chunk slots in LDS
   constexpr int kXSlot = 128 * 128;     // bytes of one slot
   constexpr int kScWave = 128;          // scale strip of a wave per slot: its 32 activation scales
-  constexpr int kMaxKC = 128;           // chunks of block scales parked in LDS (K <= 16384 bytes)
+  constexpr int kMaxKC = kMoeMaxKChunks;  // chunks of block scales parked in LDS (K <= 16384 bytes)
   constexpr int kScSlot = 4 * kScWave;
   constexpr int D = QT == 0 ? 5 : 4;    // direct-to-LDS operations per wave and chunk
-  constexpr float kScaleFloor = 1e-30f;
   __shared__ __attribute__((aligned(1024))) unsigned char x_lds[NX * kXSlot];
   __shared__ __attribute__((aligned(16))) unsigned char sc_lds[NX * kScSlot];
   __shared__ float ws_lds[4][2][kMaxKC];  // block scales of wave w's column tile ct, by chunk
@@ -428,17 +439,17 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
   // max(scale, floor) as ONE integer maximum on the bit patterns (positive floats order like
   // their bits; a negative or zero scale becomes the floor): fmaxf costs a second instruction
   // that quiets NaNs, and these sit in the main loop
-  auto floor_scale = [&](float v) -> float {
-    return __int_as_float(max(__float_as_int(v), __float_as_int(kScaleFloor)));
+  auto floor_scale = [&](float v, float floor_v) -> float {
+    return __int_as_float(max(__float_as_int(v), __float_as_int(floor_v)));
   };
   // row 32 rt + j's activation scale sits in wave rt's strip of the chunk's slot
   const unsigned char* as_mine = sc_lds + j * 4;
   auto read_as = [&](int slot, int rt) -> float {
-    return floor_scale(*(const float*)(as_mine + slot * kScSlot + rt * kScWave));
+    return floor_scale(*(const float*)(as_mine + slot * kScSlot + rt * kScWave), kActScaleFloor);
   };
   // (wave-uniform)
   auto read_ws = [&](int kc, int ct) -> float {
-    return floor_scale(ws_lds[wave][ct][kc]);
+    return floor_scale(ws_lds[wave][ct][kc], kWScaleFloor);
   };
 
   f32x16 acc[NRT][2];  // [row tile][column tile]
@@ -833,6 +844,8 @@ int fill_gemm_params(MoeGemmParams& p, bool gated, int elem, const void* a, cons
   if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
   // a row must be a whole number of 128-byte chunks; output tiles are 128 columns wide
   if ((Kel * elem) % 128 != 0 || I % 128 != 0 || H % 128 != 0) return DLB_ERR_UNSUPPORTED;
+  // fp8: the block scales of all K chunks of a tile are parked in LDS
+  if (elem == 1 && Kel / 128 > kMoeMaxKChunks) return DLB_ERR_UNSUPPORTED;
   if (!aligned16(a) || !aligned16(w)) return DLB_ERR_UNSUPPORTED;
   if ((int64_t)N * Kel * elem >= (int64_t)0xffffffffu) return DLB_ERR_UNSUPPORTED;  // 32-bit lane offsets
   const int64_t a_rows = gated ? num_tokens : (int64_t)num_mblocks * block_m;

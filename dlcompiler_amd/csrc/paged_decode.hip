@@ -31,8 +31,8 @@ struct DecodeParams {
   const void* k;
   const void* v;
   void* o;
-  const int32_t* block_table;
-  const int32_t* kv_len;
+  IdxArray block_table;
+  IdxArray kv_len;
   float* ws_o;      // [B, Hq, nsplit_max, D]
   float* ws_ml;     // [B, Hq, nsplit_max, 2]
   int32_t* ws_np;   // [B] partials written for each sequence
@@ -146,7 +146,8 @@ __global__ __launch_bounds__(64, RAGGED ? 1 : 2) void paged_decode_split_kernel(
   k_end = __builtin_amdgcn_readfirstlane(min(k_end, ctx));
   const int kv_min = p.window > 0 ? max(ctx - 1 - p.window, 0) : 0;  // first visible key
   k_begin = __builtin_amdgcn_readfirstlane(max(k_begin, kv_min & ~31));  // the half tile holding kv_min
-  const int32_t* bt = p.block_table + (int64_t)b * p.bt_stride;
+  const int32_t* bt = p.block_table.p + (((int64_t)b * p.bt_stride) << p.block_table.sh);
+  const int bt_sh = p.block_table.sh;
 
   // Q^T as the B operand: lane (n = query head c, k = dims 32*ks + 8g .. +8)
   u32x4 qf[KS];
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(64, RAGGED ? 1 : 2) void paged_decode_split_kernel(
     for (int sub = 0; sub < 2; ++sub) {
       const int base_key = min(h0 + 16 * sub, ctx - 1);  // clamp: never look past the context
       const int pi = POW2 ? (base_key >> p.page_shift) : (base_key / p.page);
-      entry[sub] = (const int32_t*)uniform_ptr((const unsigned char*)(bt + pi));
+      entry[sub] = (const int32_t*)uniform_ptr((const unsigned char*)(bt + (pi << bt_sh)));
     }
     int p0, p1;
     asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
@@ -494,8 +495,8 @@ extern "C" size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int p
 }
 
 extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache,
-                                     void* o, const int32_t* block_table, const int32_t* kv_len,
-                                     int B, int Hq, int Hkv, int D, int Dv, int page,
+                                     void* o, const void* block_table, const void* kv_len,
+                                     int index64_mask, int B, int Hq, int Hkv, int D, int Dv, int page,
                                      int max_blocks, int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_page,
                                      int64_t k_stride_tok, int64_t k_stride_head,
                                      int64_t v_stride_page, int64_t v_stride_tok,
@@ -531,8 +532,9 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   p.k = k_cache;
   p.v = v_cache;
   p.o = o;
-  p.block_table = block_table;
-  p.kv_len = kv_len;
+  if (index64_mask & ~3) return DLB_ERR_BAD_ARG;
+  p.block_table = idx_array(block_table, index64_mask, 0);
+  p.kv_len = idx_array(kv_len, index64_mask, 1);
   p.q_sb = q_stride_b;
   p.q_sh = q_stride_h;
   p.k_sp = k_stride_page;

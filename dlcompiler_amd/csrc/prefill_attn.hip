@@ -30,8 +30,8 @@ struct PrefillParams {
   const void* k;
   const void* v;
   void* o;
-  const int32_t* start_loc;
-  const int32_t* seq_len;
+  IdxArray start_loc;
+  IdxArray seq_len;
   int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;  // token / head strides (elements)
   int Hq, Hkv, group;
   int xcd_heads;  // != 0: remap blockIdx.x so the heads of a KV group share an XCD
@@ -39,8 +39,8 @@ struct PrefillParams {
   // paged K/V (PAGED kernels): k/v point at caches [pages, page, Hkv, D]; *_st is the slot
   // stride, *_sp the page stride; sequence s reads pages block_table[s][.] and its queries sit
   // at context positions kv_len[s] - seq_len[s] + i
-  const int32_t* kv_len;
-  const int32_t* block_table;
+  IdxArray kv_len;
+  IdxArray block_table;
   int64_t bt_stride, k_sp, v_sp;
   int page, page_shift;
   int dk, dv;  // real key / value head sizes (<= the padded size D the kernel is built for)
@@ -203,7 +203,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   const unsigned char* kbytes = (const unsigned char*)kb;
   const unsigned char* vbytes = (const unsigned char*)vb;
   const int64_t k_row_bytes = p.k_st * 2, v_row_bytes = p.v_st * 2;
-  const int32_t* bt = PAGED ? p.block_table + (int64_t)seq * p.bt_stride : nullptr;
+  const IdxArray bt = {PAGED ? p.block_table.p + (((int64_t)seq * p.bt_stride) << p.block_table.sh) : nullptr,
+                       p.block_table.sh};
   // V chunk swizzle of row r (depends on r mod 8 only)
   auto v_swz = [](int r) -> int {
     return D == 128 ? (((r & 3) << 2) | (((r >> 2) & 1) << 1))
@@ -550,8 +551,8 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk,
 }  // namespace dlb
 
 extern "C" int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o,
-                                       const int32_t* start_loc, const int32_t* seq_len, int B,
-                                       int Hq, int Hkv, int D, int max_len, int64_t q_stride_tok,
+                                       const void* start_loc, const void* seq_len,
+                                       int index64_mask, int B, int Hq, int Hkv, int D, int max_len, int64_t q_stride_tok,
                                        int64_t q_stride_head, int64_t k_stride_tok,
                                        int64_t k_stride_head, int64_t v_stride_tok,
                                        int64_t v_stride_head, int64_t o_stride_tok,
@@ -567,8 +568,9 @@ extern "C" int dlb_prefill_attn_varlen(const void* q, const void* k, const void*
   p.k = k;
   p.v = v;
   p.o = o;
-  p.start_loc = start_loc;
-  p.seq_len = seq_len;
+  if (index64_mask & ~3) return DLB_ERR_BAD_ARG;
+  p.start_loc = idx_array(start_loc, index64_mask, 0);
+  p.seq_len = idx_array(seq_len, index64_mask, 1);
   p.q_st = q_stride_tok;
   p.q_sh = q_stride_head;
   p.k_st = k_stride_tok;
@@ -585,9 +587,9 @@ extern "C" int dlb_prefill_attn_varlen(const void* q, const void* k, const void*
 }
 
 extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache,
-                                      void* o, const int32_t* block_table,
-                                      const int32_t* q_start_loc, const int32_t* q_len,
-                                      const int32_t* kv_len, int B, int Hq, int Hkv, int D,
+                                      void* o, const void* block_table,
+                                      const void* q_start_loc, const void* q_len,
+                                      const void* kv_len, int index64_mask, int B, int Hq, int Hkv, int D,
                                       int Dv, int page, int max_blocks, int max_q_len,
                                       int64_t q_stride_tok, int64_t q_stride_head,
                                       int64_t k_stride_page, int64_t k_stride_tok,
@@ -608,10 +610,11 @@ extern "C" int dlb_paged_prefill_attn(const void* q, const void* k_cache, const 
   p.k = k_cache;
   p.v = v_cache;
   p.o = o;
-  p.start_loc = q_start_loc;
-  p.seq_len = q_len;
-  p.kv_len = kv_len;
-  p.block_table = block_table;
+  if (index64_mask & ~15) return DLB_ERR_BAD_ARG;
+  p.block_table = idx_array(block_table, index64_mask, 0);
+  p.start_loc = idx_array(q_start_loc, index64_mask, 1);
+  p.seq_len = idx_array(q_len, index64_mask, 2);
+  p.kv_len = idx_array(kv_len, index64_mask, 3);
   p.bt_stride = bt_stride;
   p.q_st = q_stride_tok;
   p.q_sh = q_stride_head;

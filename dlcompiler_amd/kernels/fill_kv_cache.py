@@ -8,10 +8,6 @@ from torch import Tensor
 from .. import _lib
 
 
-def _i32(t: Tensor) -> Tensor:
-    return (t if t.dtype == torch.int32 else t.to(torch.int32)).contiguous()
-
-
 def fill_kv_cache(
     k_states: Tensor,
     v_states: Tensor,
@@ -25,7 +21,8 @@ def fill_kv_cache(
 ):
     """fill key/value state to cache for paged attention (in place; returns None)."""
     _lib.require_cuda(k_states, v_states, k_caches, v_caches, block_offsets)
-    block_offsets = _i32(block_offsets)
+    if block_offsets.stride(-1) != 1:
+        block_offsets = block_offsets.contiguous()
     batch_size = block_offsets.size(0)
     block_size, num_heads, head_dim = k_caches.size()[1:]
     head_dim_v = v_states.size(-1)
@@ -37,13 +34,15 @@ def fill_kv_cache(
     if num_tokens == 0 or batch_size == 0:
         return
     lib = _lib.load()
-    # converted copies must stay referenced until the launch is enqueued
-    q_start_i, q_len_i, kv_len_i = _i32(q_start_loc), _i32(q_seq_length), _i32(kv_seq_length)
+    # int32 or int64 index tensors are read as they arrive; anything converted must stay
+    # referenced until the launch is enqueued
+    (q_start_i, q_len_i, kv_len_i, block_offsets), mask = _lib.index_arrays(
+        q_start_loc.contiguous(), q_seq_length.contiguous(), kv_seq_length.contiguous(), block_offsets)
     with _lib.device_guard(k_states.device):
         st = lib.dlb_fill_kv_cache(
             k_states.data_ptr(), v_states.data_ptr(), k_caches.data_ptr(), v_caches.data_ptr(),
             q_start_i.data_ptr(), q_len_i.data_ptr(), kv_len_i.data_ptr(),
-            block_offsets.data_ptr(), num_tokens, batch_size,
+            block_offsets.data_ptr(), mask, num_tokens, batch_size,
             num_heads, head_dim, head_dim_v, block_size, block_offsets.size(1),
             k_states.element_size(), k_states.stride(0), k_states.stride(1), v_states.stride(0),
             v_states.stride(1), k_caches.stride(0), k_caches.stride(1), k_caches.stride(2),

@@ -8,10 +8,6 @@ from torch import Tensor
 from .. import _lib
 
 
-def _as_int32(t: Tensor) -> Tensor:
-    return t if t.dtype == torch.int32 else t.to(torch.int32)
-
-
 def paged_attention_fwd(
     q: Tensor,
     k: Tensor,
@@ -56,24 +52,23 @@ def paged_attention_fwd(
     num_kv_heads = k.shape[-2]
     assert head % num_kv_heads == 0
     page = k.size(1)
-    assert page >= 16
     for t in (q, k, v, o):
         assert t.stride(-1) == 1, "last dimension must be contiguous"
-    block_offsets = _as_int32(block_offsets)
+    # the index tensors are read in the integer width they arrive in (int32 or int64), as the
+    # reference's kernels do (paged_attention.py:492-559): no per-call conversion launches
     if block_offsets.stride(-1) != 1:
         block_offsets = block_offsets.contiguous()
-    kv_seqlens = _as_int32(kv_seqlens).contiguous()
     max_blocks = block_offsets.size(1)
     lib = _lib.load()
 
     if not is_decoding:
         assert q.dim() == 3 and o.dim() == 3
-        q_start_loc = _as_int32(q_start_loc).contiguous()
-        q_seqlens = _as_int32(q_seqlens).contiguous()
+        (block_offsets, q_start_loc, q_seqlens, kv_seqlens), mask = _lib.index_arrays(
+            block_offsets, q_start_loc.contiguous(), q_seqlens.contiguous(), kv_seqlens.contiguous())
         with _lib.device_guard(q.device):
             st = lib.dlb_paged_prefill_attn(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), block_offsets.data_ptr(),
-                q_start_loc.data_ptr(), q_seqlens.data_ptr(), kv_seqlens.data_ptr(), batch, head,
+                q_start_loc.data_ptr(), q_seqlens.data_ptr(), kv_seqlens.data_ptr(), mask, batch, head,
                 num_kv_heads, Lq, Lv, page, max_blocks, int(max_seqlen), q.stride(0), q.stride(1),
                 k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
                 o.stride(0), o.stride(1), block_offsets.stride(0), float(sm_scale),
@@ -82,6 +77,9 @@ def paged_attention_fwd(
         _lib.check(st, "dlb_paged_prefill_attn")
         return
 
+    if page % 16 != 0:
+        raise NotImplementedError("the decode kernel needs a page size that is a multiple of 16")
+    (block_offsets, kv_seqlens), mask = _lib.index_arrays(block_offsets, kv_seqlens.contiguous())
     q3 = q.reshape(batch, head, Lq) if q.dim() != 3 else q
     o3 = o.reshape(batch, head, Lv) if o.dim() != 3 else o
     assert o3.data_ptr() == o.data_ptr()
@@ -90,7 +88,7 @@ def paged_attention_fwd(
     with _lib.device_guard(q.device):
         st = lib.dlb_paged_decode_attn(
             q3.data_ptr(), k.data_ptr(), v.data_ptr(), o3.data_ptr(), block_offsets.data_ptr(),
-            kv_seqlens.data_ptr(), batch, head, num_kv_heads, Lq, Lv, page, max_blocks,
+            kv_seqlens.data_ptr(), mask, batch, head, num_kv_heads, Lq, Lv, page, max_blocks,
             q3.stride(0), q3.stride(1), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), o3.stride(0), o3.stride(1),
             block_offsets.stride(0), float(sm_scale), int(window_size), float(logit_softcapping),

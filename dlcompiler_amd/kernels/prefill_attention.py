@@ -7,11 +7,6 @@ import torch
 from .. import _lib
 
 
-def _as_int32(t: torch.Tensor) -> torch.Tensor:
-    t = t if t.dtype == torch.int32 else t.to(torch.int32)
-    return t.contiguous()
-
-
 def context_attention_fwd(q, k, v, o, b_start_loc, b_seq_len, max_input_len):
     """Causal attention over packed variable-length sequences, written into ``o``.
 
@@ -32,12 +27,13 @@ def context_attention_fwd(q, k, v, o, b_start_loc, b_seq_len, max_input_len):
     if batch == 0 or q.shape[0] == 0:
         return
     lib = _lib.load()
-    start = _as_int32(b_start_loc)
-    lens = _as_int32(b_seq_len)
+    # int32 or int64, read as they arrive (the reference's kernel loads them in their own type,
+    # prefill_attention.py:155-181)
+    (start, lens), mask = _lib.index_arrays(b_start_loc.contiguous(), b_seq_len.contiguous())
     with _lib.device_guard(q.device):
         st = lib.dlb_prefill_attn_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), start.data_ptr(),
-            lens.data_ptr(), batch, head, k.shape[1], Lq, int(max_input_len),
+            lens.data_ptr(), mask, batch, head, k.shape[1], Lq, int(max_input_len),
             q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
             o.stride(0), o.stride(1), float(sm_scale), _lib.torch_dtype_code(q.dtype),
             _lib.current_stream_ptr(q.device))

@@ -35,8 +35,15 @@ extern "C" {
 #define DLB_DTYPE_F16 1
 #define DLB_DTYPE_F32 2
 
-/* ABI version: bumped whenever a signature below changes. */
+/* ABI version: bumped whenever a signature below changes; dlb_version() returns the value the
+ * library was built with, and a binding should refuse a library whose version differs. */
+#define DLB_ABI_VERSION 3
 int dlb_version(void);
+
+/* Index arrays (block tables, sequence lengths, start offsets) are read in the integer width the
+ * caller's framework holds them in: every entry point that takes such arrays has an
+ * `index64_mask` argument whose bit i is set when the i-th index array of its signature (in
+ * argument order) holds int64 instead of int32.  Values must lie in [0, 2^31). */
 /* static string for a status code (never NULL). */
 const char* dlb_status_string(int status);
 
@@ -99,7 +106,9 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
  * process ends.  Limit: numel <= dlb_moe_align_block_size_static_max_numel() (524288 routing
  * slots); more returns DLB_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls
  * that overlap on one GPU (different streams) race; calls on one stream are ordered.  Nothing
- * in the array has to be cleared between calls.
+ * in the array has to be cleared between calls.  The first call on a device looks up the array's
+ * address there (hipGetSymbolAddress, which may load the library's device code): make one call on
+ * every device outside stream capture before the entry point is used in a captured region.
  * ---------------------------------------------------------------------------------------- */
 int64_t dlb_moe_align_block_size_static_max_numel(void);
 int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int E, int block,
@@ -132,8 +141,11 @@ int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t*
  *   k cache      [pages, page, Hkv, D] strides k_stride_page, k_stride_tok, k_stride_head
  *   v cache      [pages, page, Hkv, Dv] strides v_stride_page, v_stride_tok, v_stride_head
  *   o            [B, Hq, Dv]           strides o_stride_b, o_stride_h
- *   block_table  int32 [B, max_blocks] row stride bt_stride: physical page of logical page j
- *   kv_len       int32 [B]             context length; rows with kv_len <= 0 produce zeros
+ *   block_table  int32/int64 [B, max_blocks] row stride bt_stride (elements): physical page of
+ *                logical page j (index64_mask bit 0)
+ *   kv_len       int32/int64 [B]       context length; rows with kv_len <= 0 produce zeros
+ *                (index64_mask bit 1); the reference reads both in whatever integer type arrives,
+ *                kernels/paged_attention.py:492-559
  * out[b, h] = softmax(q[b, h] . K[b, h / (Hq/Hkv)]^T * sm_scale) V, softmax in fp32 and P
  * rounded to `dtype` before P.V, as in the reference.
  * window_size > 0 masks keys older than kv_len - 1 - window_size (sliding window,
@@ -148,8 +160,8 @@ int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t*
  * ---------------------------------------------------------------------------------------- */
 size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int page, int max_blocks);
 int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, void* o,
-                          const int32_t* block_table, const int32_t* kv_len, int B, int Hq,
-                          int Hkv, int D, int Dv, int page, int max_blocks, int64_t q_stride_b,
+                          const void* block_table, const void* kv_len, int index64_mask, int B,
+                          int Hq, int Hkv, int D, int Dv, int page, int max_blocks, int64_t q_stride_b,
                           int64_t q_stride_h, int64_t k_stride_page, int64_t k_stride_tok,
                           int64_t k_stride_head, int64_t v_stride_page, int64_t v_stride_tok,
                           int64_t v_stride_head, int64_t o_stride_b, int64_t o_stride_h,
@@ -162,7 +174,8 @@ int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cach
  * Replaces context_attention_fwd + _fwd_kernel, kernels/prefill_attention.py:39-181.
  *   q [tokens, Hq, D], k/v [tokens, Hkv, D], o [tokens, Hq, D]; token and head strides given,
  *   unit stride in D.  Sequence s owns tokens start_loc[s] .. start_loc[s] + seq_len[s] - 1
- *   (int32 [B] each; with cu_seqlens: start_loc = cu[:-1], seq_len = cu[1:] - cu[:-1]).
+ *   (int32 or int64 [B] each: index64_mask bit 0 = start_loc, bit 1 = seq_len; with cu_seqlens:
+ *   start_loc = cu[:-1], seq_len = cu[1:] - cu[:-1]).
  *   max_len >= max(seq_len) sizes the grid (the reference's max_input_len).
  * o[t, h] = sum_{t' <= t, same sequence} softmax_t'(q[t, h] . k[t', h / (Hq/Hkv)] * sm_scale)
  *           v[t', h / (Hq/Hkv)], softmax in fp32, P rounded to `dtype` before P.V.
@@ -173,8 +186,8 @@ int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cach
  * sequence are not written.
  * ---------------------------------------------------------------------------------------- */
 int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o,
-                            const int32_t* start_loc, const int32_t* seq_len, int B, int Hq,
-                            int Hkv, int D, int max_len, int64_t q_stride_tok,
+                            const void* start_loc, const void* seq_len, int index64_mask, int B,
+                            int Hq, int Hkv, int D, int max_len, int64_t q_stride_tok,
                             int64_t q_stride_head, int64_t k_stride_tok, int64_t k_stride_head,
                             int64_t v_stride_tok, int64_t v_stride_head, int64_t o_stride_tok,
                             int64_t o_stride_head, float sm_scale, int dtype, void* stream);
@@ -186,9 +199,9 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
  * kernels/paged_attention.py:319-489, 559-607.
  *   q [tokens, Hq, D], o [tokens, Hq, Dv]: sequence s owns query tokens q_start_loc[s] ..
  *   q_start_loc[s] + q_len[s] - 1; k_cache [pages, page, Hkv, D], v_cache [pages, page, Hkv, Dv];
- *   block_table int32
- *   [B, max_blocks]; kv_len int32 [B] = history + q_len[s] (sequences with kv_len < q_len are
- *   skipped).  Query i of sequence s sits at context position kv_len[s] - q_len[s] + i and
+ *   block_table [B, max_blocks]; kv_len [B] = history + q_len[s] (sequences with kv_len < q_len
+ *   are skipped); the four index arrays are int32 or int64 (index64_mask bit 0 = block_table,
+ *   1 = q_start_loc, 2 = q_len, 3 = kv_len).  Query i of sequence s sits at context position kv_len[s] - q_len[s] + i and
  *   sees keys 0 .. that position (paged_attention.py:455), or, with window_size > 0, only the
  *   keys >= position - window_size (:429-431,457-458); logit_softcapping > 0 replaces the
  *   scaled logits by cap * tanh(logits / cap) (:450-453).  Pass <= 0 to disable either.
@@ -198,8 +211,8 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
  * aligned, o strides multiples of 4 and base 8-byte aligned.
  * ---------------------------------------------------------------------------------------- */
 int dlb_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, void* o,
-                           const int32_t* block_table, const int32_t* q_start_loc,
-                           const int32_t* q_len, const int32_t* kv_len, int B, int Hq, int Hkv,
+                           const void* block_table, const void* q_start_loc, const void* q_len,
+                           const void* kv_len, int index64_mask, int B, int Hq, int Hkv,
                            int D, int Dv, int page, int max_blocks, int max_q_len,
                            int64_t q_stride_tok,
                            int64_t q_stride_head, int64_t k_stride_page, int64_t k_stride_tok,
@@ -240,7 +253,10 @@ int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs, int64_t M,
  *   hq [num_mblocks * block_m, I] fp8 and hs [num_mblocks * block_m, I/128]: row r holds
  *     quant(silu(x_t W_gate^T) * (x_t W_up^T)) for the slot at sorted position r (rows of
  *     32-row groups that hold padding only are not written)
- * H % 128 == 0, I % 128 == 0; scales must be positive (values below 1e-30 count as 1e-30).
+ * H % 128 == 0, I % 128 == 0, and the reduction length (H here, I in the down GEMM) at most
+ * 16384.  Scales must be positive: activation scales below 1e-13 count as 1e-13 (the quantisation
+ * rule above never produces less than 1e-10 / 448) and weight block scales below 1e-12 count as
+ * 1e-12 (an all-zero block may carry the scale 0).
  * One kernel serves both tile heights and both weight layouts: four-wave tiles of block_m rows
  * x 256 columns, weights streamed straight into operand registers, activations staged in LDS.
  * Outputs are stored 16 bytes at a time: hq, out and the 16-bit act must be 16-byte aligned;
@@ -310,11 +326,12 @@ int dlb_moe_gemm_16bit_down(const void* act, const void* w2, const int32_t* sort
  *   sequence b owns tokens q_start_loc[b] .. + q_seq_len[b]; its i-th new token lands at
  *   context position kv_seq_len[b] - q_seq_len[b] + i, i.e. page
  *   block_table[b][pos / page], slot pos % page.  Tokens outside every sequence are ignored.
+ *   The four index arrays are int32 or int64 (index64_mask bit 0 = q_start_loc, 1 = q_seq_len,
+ *   2 = kv_seq_len, 3 = block_table).
  * elem_size = bytes per element (the copy is type-agnostic); strides in elements. */
 int dlb_fill_kv_cache(const void* k_states, const void* v_states, void* k_cache, void* v_cache,
-                      const int32_t* q_start_loc, const int32_t* q_seq_len,
-                      const int32_t* kv_seq_len, const int32_t* block_table, int64_t num_tokens,
-                      int batch, int heads, int head_dim, int head_dim_v, int page, int max_blocks,
+                      const void* q_start_loc, const void* q_seq_len, const void* kv_seq_len,
+                      const void* block_table, int index64_mask, int64_t num_tokens, int batch, int heads, int head_dim, int head_dim_v, int page, int max_blocks,
                       int elem_size, int64_t ks_stride_tok, int64_t ks_stride_head,
                       int64_t vs_stride_tok, int64_t vs_stride_head, int64_t kc_stride_page,
                       int64_t kc_stride_slot, int64_t kc_stride_head, int64_t vc_stride_page,
@@ -340,22 +357,6 @@ int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void* cos, cons
                              int64_t k_stride_head, int64_t qo_stride_tok, int64_t qo_stride_head,
                              int64_t ko_stride_tok, int64_t ko_stride_head, int64_t cs_stride_tok,
                              int dtype, void* stream);
-
-/* Measurement aid (no counterpart in the reference; used by bench.py, not by any operator):
- * launches `blocks` workgroups of 512 threads that each issue `iters` rounds of four independent
- * MFMAs per wave (bf16 32x32x16, or fp8 32x32x64 when fp8 != 0) on operand registers loaded once
- * from `operands` -- no memory traffic, LDS or vector arithmetic in the loop.  Timed by the
- * caller, it gives the matrix rate this chip sustains on that operand DATA (the clock under
- * matrix load follows the power the data draws).  FLOPs = blocks * 8 waves * iters * 4 * (32768
- * for bf16, 131072 for fp8).  operands: at least dlb_probe_mfma_operand_bytes(blocks) bytes,
- * 16-byte aligned, any contents; sink: 2 KB the kernel practically never writes. */
-int64_t dlb_probe_mfma_operand_bytes(int blocks);
-/* Second measurement aid: reads `bytes` (a multiple of 16) from src with non-temporal 16-byte
- * loads, eight in flight per lane, and discards them.  Timed by the caller it is the HBM rate a
- * kernel with no arithmetic and no stores reaches on this chip. */
-int dlb_probe_hbm_read(const void* src, void* sink, int64_t bytes, void* stream);
-int dlb_probe_mfma_rate(const void* operands, int64_t operand_bytes, void* sink, int blocks,
-                        int fp8, int iters, void* stream);
 
 #ifdef __cplusplus
 }

@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_status_strings():
     lib = _lib.load()
-    assert lib.dlb_version() >= 1
+    assert lib.dlb_version() == _lib.ABI_VERSION == 3
     assert lib.dlb_status_string(0) == b"ok"
     for code in (-1, -2, -3, -4, -99):
         assert lib.dlb_status_string(code)
@@ -74,6 +74,7 @@ def test_moe_gemm_argument_checks_need_no_gpu():
     assert gate_up(num_mblocks=0) == 0                    # nothing to do
     assert gate_up(block_m=96) == -2                      # tile heights are 64 and 128
     assert gate_up(H=200) == -2                           # rows are whole 128-byte chunks
+    assert gate_up(H=16512) == -2                         # more than 128 chunks of block scales
     assert gate_up(num_experts=300, local=300) == -2      # at most 256 experts
     assert gate_up(offset=4, local=8) == -1               # local experts must lie inside the global range
     assert gate_up(num_mblocks=-1) == -1

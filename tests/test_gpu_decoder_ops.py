@@ -16,7 +16,8 @@ def _div_up(a, b):
                                                    ((1, 8, 16, 24), (1, 16, 31, 24)),
                                                    ((70, 1, 130), (0, 63, 64))])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_fill_kv_cache(dev, seq_lens, history_lens, dtype):
+@pytest.mark.parametrize("idx", [torch.int64, torch.int32, "mixed"])
+def test_fill_kv_cache(dev, seq_lens, history_lens, dtype, idx):
     from dlcompiler_amd.kernels.fill_kv_cache import fill_kv_cache
 
     g = torch.Generator().manual_seed(0)
@@ -33,8 +34,10 @@ def test_fill_kv_cache(dev, seq_lens, history_lens, dtype):
     q_start = q_len.cumsum(0) - q_len
     rk, rv = od.fill_kv_cache(ks, vs, kc, vc, seq_lens, history_lens, table)
     kcd, vcd = kc.to(dev), vc.to(dev)
-    fill_kv_cache(ks.to(dev), vs.to(dev), kcd, vcd, q_start.to(dev), q_len.to(dev),
-                  torch.tensor(kv_lens).to(dev), max(seq_lens), table.to(dev))
+    # index tensors are read in the integer width they arrive in
+    it = [torch.int64, torch.int32, torch.int16, torch.int32] if idx == "mixed" else [idx] * 4
+    fill_kv_cache(ks.to(dev), vs.to(dev), kcd, vcd, q_start.to(it[0]).to(dev), q_len.to(it[1]).to(dev),
+                  torch.tensor(kv_lens).to(it[2]).to(dev), max(seq_lens), table.to(it[3]).to(dev))
     assert torch.equal(kcd.cpu(), rk) and torch.equal(vcd.cpu(), rv)     # a copy: exact
 
 

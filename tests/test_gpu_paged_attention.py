@@ -12,7 +12,7 @@ def _rand(shape, seed, dtype):
 
 
 def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_dtype=torch.int32,
-              sm_scale=None, uniform=False, window=None, softcap=None, dv=None):
+              sm_scale=None, uniform=False, window=None, softcap=None, dv=None, len_dtype=torch.int64):
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
     if uniform:   # the reference test draws torch.rand inputs (test_paged_attention.py:157-180)
@@ -31,7 +31,7 @@ def _run_case(dev, lens, hq, hkv, d, page, dtype, seed=0, num_pages=None, table_
     o = torch.full((B, hq, dv), 9.0, dtype=dtype, device=dev)
     ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(table_dtype).to(dev),
                               torch.arange(B, device=dev), torch.ones(B, dtype=torch.int64, device=dev),
-                              kv_len.to(dev), 1, sm_scale=sm_scale, window_size=window,
+                              kv_len.to(len_dtype).to(dev), 1, sm_scale=sm_scale, window_size=window,
                               logit_softcapping=softcap)
     assert ret is None
     out = o.cpu()
@@ -58,6 +58,19 @@ def test_reference_decode_cases(dev, hq, hkv, d, dv):
 def test_context_length_edges(dev, dtype, page):
     lens = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 511, 512, 513, 1000, 0]
     _run_case(dev, lens, 32, 8, 128, page, dtype)
+
+
+# block table and context lengths are read in the integer width they arrive in
+@pytest.mark.parametrize("table_dtype,len_dtype", [(torch.int32, torch.int32), (torch.int64, torch.int64),
+                                                   (torch.int32, torch.int64), (torch.int64, torch.int32),
+                                                   (torch.int16, torch.int16)])
+def test_index_dtypes(dev, table_dtype, len_dtype):
+    lens = [1, 17, 300, 1025, 64, 0, 2049]
+    out, _ = _run_case(dev, lens, 32, 8, 128, 16, torch.bfloat16, table_dtype=table_dtype,
+                       len_dtype=len_dtype)
+    ref32, _ = _run_case(dev, lens, 32, 8, 128, 16, torch.bfloat16)
+    assert torch.equal(out, ref32)
+    _run_case(dev, [513, 77], 8, 2, 64, 48, torch.float16, table_dtype=table_dtype, len_dtype=len_dtype)
 
 
 def test_group_sizes_and_scale(dev):
@@ -138,6 +151,11 @@ def test_unsupported_requests_raise(dev):
         paged_attention_fwd(*args(44))                       # head size not a multiple of 8
     with pytest.raises(NotImplementedError):
         paged_attention_fwd(*args(136))                      # head size above 128
+    q = torch.zeros((2, 4, 64), dtype=torch.float16, device=dev)
+    kc = torch.zeros((4, 8, 2, 64), dtype=torch.float16, device=dev)
+    with pytest.raises(NotImplementedError):                 # decode pages are multiples of 16
+        paged_attention_fwd(q, kc, kc, torch.zeros_like(q), torch.zeros((2, 2), dtype=torch.int32, device=dev),
+                            None, torch.ones(2, device=dev), torch.tensor([3, 4], device=dev), 1)
 
 
 def test_config4_full(dev):

@@ -9,7 +9,9 @@ pytestmark = pytest.mark.gpu
 
 
 def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False, window=None,
-              softcap=None, sm_scale=None, max_seqlen=None, tol=2e-2, dv=None):
+              softcap=None, sm_scale=None, max_seqlen=None, tol=2e-2, dv=None,
+              idx_dtypes=(torch.int64,) * 4):
+    # idx_dtypes: integer types of (block_offsets, q_start_loc, q_seqlens, kv_seqlens) as handed over
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
     gen = torch.Generator().manual_seed(123 + seed)
@@ -29,8 +31,10 @@ def _run_case(dev, q_lens, hist, hq, hkv, d, page, dtype, seed=0, uniform=False,
     ref = oa.paged_prefill(q, kc, vc, table, start, ql, kl, sm_scale=sm_scale, window=window,
                            softcap=softcap)
     o = torch.full((T + 3, hq, dv), 9.0, dtype=dtype, device=dev)
-    ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(dev), start.to(dev),
-                              ql.to(dev), kl.to(dev), max_seqlen or max(q_lens),
+    it = idx_dtypes
+    ret = paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o, table.to(it[0]).to(dev),
+                              start.to(it[1]).to(dev), ql.to(it[2]).to(dev), kl.to(it[3]).to(dev),
+                              max_seqlen or max(q_lens),
                               window_size=window, sm_scale=sm_scale, logit_softcapping=softcap)
     assert ret is None
     out = o.cpu()
@@ -111,6 +115,28 @@ def test_large_chunked_prefill(dev):
 def test_odd_page_sizes(dev, page):
     _run_case(dev, [70, 33, 129], [45, 0, 200], 4, 2, 128, page, torch.bfloat16, seed=page)
     _run_case(dev, [65], [130], 2, 1, 64, page, torch.float16, seed=page + 1, window=40)
+
+
+# the prefill branch looks up the page of every K/V row, so any page size works, down to one
+# token per page (the decode branch needs multiples of 16)
+@pytest.mark.parametrize("page", [1, 4, 8])
+def test_small_pages(dev, page):
+    _run_case(dev, [70, 33, 129, 1], [45, 0, 200, 7], 4, 2, 128, page, torch.bfloat16, seed=page)
+    _run_case(dev, [65, 5], [130, 3], 2, 1, 64, page, torch.float16, seed=page + 1, window=40)
+
+
+# the index tensors are read in the integer width they arrive in: all int32, all int64 (what
+# lmdeploy hands over), mixtures, and a narrower type that the wrapper converts
+@pytest.mark.parametrize("idx", [(torch.int32,) * 4, (torch.int64,) * 4,
+                                 (torch.int64, torch.int32, torch.int64, torch.int32),
+                                 (torch.int32, torch.int64, torch.int32, torch.int64),
+                                 (torch.int16, torch.int64, torch.int16, torch.int32)])
+def test_index_dtypes(dev, idx):
+    out = [_run_case(dev, [30, 129, 64], [50, 300, 0], 8, 2, 128, 16, torch.bfloat16, seed=11,
+                     idx_dtypes=idx)[0]]
+    ref32 = _run_case(dev, [30, 129, 64], [50, 300, 0], 8, 2, 128, 16, torch.bfloat16, seed=11,
+                      idx_dtypes=(torch.int32,) * 4)[0]
+    assert torch.equal(out[0], ref32)                     # same kernel, same bits
 
 
 def test_grid_larger_than_needed_and_rejects(dev):

@@ -12,7 +12,8 @@ def _rand(shape, seed, dtype, mean=0.0, std=1.0):
     return x.to(dtype)
 
 
-def _run(dev, lens, hq, hkv, d, dtype, stats=((0, 1), (0, 1), (0, 1)), gap=0, atol=2e-2, rtol=2e-2):
+def _run(dev, lens, hq, hkv, d, dtype, stats=((0, 1), (0, 1), (0, 1)), gap=0, atol=2e-2, rtol=2e-2,
+         idx_dtypes=(torch.int32, torch.int32)):
     from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
 
     starts, at = [], 0
@@ -27,8 +28,8 @@ def _run(dev, lens, hq, hkv, d, dtype, stats=((0, 1), (0, 1), (0, 1)), gap=0, at
     seqlen = torch.tensor(lens, dtype=torch.int32)
     ref = oa.prefill_attention(q, k, v, start, seqlen)
     o = torch.full((total, hq, d), 5.0, dtype=dtype, device=dev)
-    ret = context_attention_fwd(q.to(dev), k.to(dev), v.to(dev), o, start.to(dev), seqlen.to(dev),
-                                max(lens) if lens else 0)
+    ret = context_attention_fwd(q.to(dev), k.to(dev), v.to(dev), o, start.to(idx_dtypes[0]).to(dev),
+                                seqlen.to(idx_dtypes[1]).to(dev), max(lens) if lens else 0)
     assert ret is None
     out = o.cpu()
     inside = torch.zeros(total, dtype=torch.bool)
@@ -51,6 +52,16 @@ def test_reference_case(dev):
 def test_length_edges_gqa(dev, dtype, d):
     lens = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 700]
     _run(dev, lens, 8, 2, d, dtype)
+
+
+# b_start_loc / b_seq_len are read in the integer width they arrive in
+@pytest.mark.parametrize("idx", [(torch.int64, torch.int64), (torch.int32, torch.int64),
+                                 (torch.int64, torch.int32), (torch.int16, torch.uint8)])
+def test_index_dtypes(dev, idx):
+    lens = [5, 130, 64, 200]
+    out, _ = _run(dev, lens, 8, 2, 128, torch.bfloat16, gap=3, idx_dtypes=idx)
+    ref32, _ = _run(dev, lens, 8, 2, 128, torch.bfloat16, gap=3)
+    assert torch.equal(out, ref32)
 
 
 def test_group_sizes(dev):

@@ -30,14 +30,23 @@ def _align_pair(ids, E, block):
                                       ws.data_ptr(), ws.numel() * 4, stream)
     assert st == 0
     _, _, s1, e1, c1, n1 = _buffers(numel, E, block, dev)
-    torch.cuda.synchronize()
+
+    def call_static():
+        st = lib.dlb_moe_align_block_size_static(ids.data_ptr(), numel, E, block, s1.data_ptr(), cap,
+                                                 e1.data_ptr(), nblk, c1.data_ptr(), n1.data_ptr(),
+                                                 stream)
+        assert st == 0
+        torch.cuda.synchronize()
+
+    # first call on this device: the module's code object and the address of the static array are
+    # looked up here, once; the call after it must leave the device's free memory as it found it
+    # (hipMemGetInfo sees every allocation, not only those of torch's caching allocator)
+    call_static()
     before = torch.cuda.memory_allocated(dev)
-    st = lib.dlb_moe_align_block_size_static(ids.data_ptr(), numel, E, block, s1.data_ptr(), cap,
-                                             e1.data_ptr(), nblk, c1.data_ptr(), n1.data_ptr(),
-                                             stream)
-    assert st == 0
-    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    call_static()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
     return (s0, e0, c0, n0), (s1, e1, c1, n1)
 
 
