@@ -23,8 +23,8 @@ SIGNATURES = {
     "dlb_status_string": (c_char_p, [c_int]),
     "dlb_silu_and_mul": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int,
                                  c_void_p]),
-    "dlb_moe_topk_softmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,
-                                         c_int64, c_int, c_void_p]),
+    "dlb_moe_topk_softmax_f32": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int64, c_int,
+                                                          c_void_p]),
     "dlb_moe_align_ws_bytes": (c_size_t, [c_int64, c_int]),
     "dlb_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                          c_void_p, c_int64, c_void_p, c_void_p, c_void_p,

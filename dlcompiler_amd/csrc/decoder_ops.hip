@@ -290,6 +290,76 @@ __global__ __launch_bounds__(256) void rotary_f32_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Element-wise variants for shapes the vector kernels do not take: rows of any length and any
+// alignment (rms_norm; the reference masks `offsets < N_COLS`, rms_norm.py:8-75) and any even
+// head size (rotary).  Same arithmetic and rounding points, one element per thread and step.
+// ---------------------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ float ld_elem(const void* p, int64_t i) {
+  if constexpr (DT == DLB_DTYPE_F32) return ((const float*)p)[i];
+  else return Elem<DT>::load1(p, i);
+}
+template <int DT>
+__device__ __forceinline__ void st_elem(void* p, int64_t i, float v) {
+  if constexpr (DT == DLB_DTYPE_F32) ((float*)p)[i] = v;
+  else Elem<DT>::store1(p, i, v);
+}
+// v rounded to the storage type
+template <int DT>
+__device__ __forceinline__ float round_elem(float v) {
+  if constexpr (DT == DLB_DTYPE_F32) return v;
+  else return Elem<DT>::lo(Elem<DT>::pack(v, 0.0f));
+}
+
+template <int DT, bool ADD>
+__global__ __launch_bounds__(kNormThreads) void rms_norm_any_kernel(
+    const void* __restrict__ x, const void* __restrict__ w, const void* __restrict__ res,
+    void* __restrict__ out, void* __restrict__ out_res, int N, int64_t ld_x, int64_t ld_res,
+    int64_t ld_out, int64_t ld_out_res, float eps) {
+  __shared__ float red[kNormThreads / 64];
+  const int64_t row = blockIdx.x;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < N; i += kNormThreads) {
+    float v = ld_elem<DT>(x, row * ld_x + i);
+    if (ADD) {
+      v = round_elem<DT>(v + ld_elem<DT>(res, row * ld_res + i));
+      st_elem<DT>(out_res, row * ld_out_res + i, v);  // read back below by the thread that wrote it
+    }
+    ss += v * v;
+  }
+  const float var = block_sum(ss, red) / (float)N;
+  const float inv = rsqrtf(var + eps);
+  for (int i = threadIdx.x; i < N; i += kNormThreads) {
+    const float v = ADD ? ld_elem<DT>(out_res, row * ld_out_res + i) : ld_elem<DT>(x, row * ld_x + i);
+    st_elem<DT>(out, row * ld_out + i, round_elem<DT>(v * inv) * ld_elem<DT>(w, i));
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void rotary_any_kernel(
+    const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ cos_,
+    const void* __restrict__ sin_, void* qo, void* ko, int Hq, int Hk, int D, int64_t q_st,
+    int64_t q_sh, int64_t k_st, int64_t k_sh, int64_t qo_st, int64_t qo_sh, int64_t ko_st,
+    int64_t ko_sh, int64_t cs_st) {
+  const int64_t t = blockIdx.x;
+  const int half = D >> 1;
+  const int total = (Hq + Hk) * half;
+  for (int u = threadIdx.x; u < total; u += 256) {
+    const int h = u / half, d = u - h * half;
+    const void* src = h < Hq ? q : k;
+    void* dst = h < Hq ? qo : ko;
+    const int64_t so = h < Hq ? t * q_st + (int64_t)h * q_sh : t * k_st + (int64_t)(h - Hq) * k_sh;
+    const int64_t dof = h < Hq ? t * qo_st + (int64_t)h * qo_sh : t * ko_st + (int64_t)(h - Hq) * ko_sh;
+    // both halves are read before either is written: in place is allowed
+    const float xl = ld_elem<DT>(src, so + d), xh = ld_elem<DT>(src, so + half + d);
+    const float cl = ld_elem<DT>(cos_, t * cs_st + d), ch = ld_elem<DT>(cos_, t * cs_st + half + d);
+    const float sl = ld_elem<DT>(sin_, t * cs_st + d), sh = ld_elem<DT>(sin_, t * cs_st + half + d);
+    st_elem<DT>(dst, dof + d, xl * cl - xh * sl);
+    st_elem<DT>(dst, dof + half + d, xh * ch + xl * sh);
+  }
+}
+
 inline bool mult16(int64_t v) { return (v & 15) == 0; }
 
 }  // namespace
@@ -365,15 +435,33 @@ extern "C" int dlb_rms_norm(const void* x, const void* weight, const void* resid
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16 && dtype != DLB_DTYPE_F32)
     return DLB_ERR_UNSUPPORTED;
   const int vec = dtype == DLB_DTYPE_F32 ? 4 : 8;  // elements per 16-byte vector
-  if (N % vec != 0 || N > kNormThreads * kMaxVec * 8) return DLB_ERR_UNSUPPORTED;
-  if (ld_x % vec != 0 || ld_out % vec != 0 || !aligned16(x) || !aligned16(weight) || !aligned16(out))
-    return DLB_ERR_UNSUPPORTED;
-  if (residual && (ld_res % vec != 0 || ld_out_res % vec != 0 || !aligned16(residual) ||
-                   !aligned16(out_residual)))
-    return DLB_ERR_UNSUPPORTED;
+  if (ld_x < N || ld_out < N || (residual && (ld_res < N || ld_out_res < N))) return DLB_ERR_BAD_ARG;
   if (M > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)M), block(kNormThreads);
+  // the vector kernels keep a row of up to 16384 elements in registers and move 16-byte pieces;
+  // any other row length or alignment takes the element-wise kernel
+  bool vector_ok = N % vec == 0 && N <= kNormThreads * kMaxVec * 8 && ld_x % vec == 0 &&
+                   ld_out % vec == 0 && aligned16(x) && aligned16(weight) && aligned16(out);
+  if (residual)
+    vector_ok = vector_ok && ld_res % vec == 0 && ld_out_res % vec == 0 && aligned16(residual) &&
+                aligned16(out_residual);
+  if (!vector_ok) {
+#define DLB_LAUNCH_NORM_ANY(DT_)                                                                   \
+  do {                                                                                             \
+    if (residual)                                                                                  \
+      hipLaunchKernelGGL((rms_norm_any_kernel<DT_, true>), grid, block, 0, s, x, weight, residual, \
+                         out, out_residual, N, ld_x, ld_res, ld_out, ld_out_res, eps);             \
+    else                                                                                           \
+      hipLaunchKernelGGL((rms_norm_any_kernel<DT_, false>), grid, block, 0, s, x, weight, residual, \
+                         out, out_residual, N, ld_x, ld_res, ld_out, ld_out_res, eps);             \
+  } while (0)
+    if (dtype == DLB_DTYPE_F32) DLB_LAUNCH_NORM_ANY(DLB_DTYPE_F32);
+    else if (dtype == DLB_DTYPE_BF16) DLB_LAUNCH_NORM_ANY(DLB_DTYPE_BF16);
+    else DLB_LAUNCH_NORM_ANY(DLB_DTYPE_F16);
+#undef DLB_LAUNCH_NORM_ANY
+    return launch_status();
+  }
   static_assert(kMaxVecF32 * 4 == kMaxVec * 8, "same row length limit for every element type");
   if (dtype == DLB_DTYPE_F32) {
     if (residual)
@@ -417,16 +505,25 @@ extern "C" int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16 && dtype != DLB_DTYPE_F32)
     return DLB_ERR_UNSUPPORTED;
   const int vec = dtype == DLB_DTYPE_F32 ? 4 : 8;  // elements per 16-byte vector
-  if (D % (2 * vec) != 0 || num_tokens > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
+  if (D % 2 != 0 || num_tokens > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
   const int64_t strides[] = {q_stride_tok,  q_stride_head,  k_stride_tok,  k_stride_head, qo_stride_tok,
                              qo_stride_head, ko_stride_tok, ko_stride_head, cs_stride_tok};
-  for (int64_t sd : strides)
-    if (sd % vec != 0) return DLB_ERR_UNSUPPORTED;
-  if (!aligned16(q) || !aligned16(k) || !aligned16(cos) || !aligned16(sin) || !aligned16(q_out) ||
-      !aligned16(k_out))
-    return DLB_ERR_UNSUPPORTED;
+  bool vector_ok = D % (2 * vec) == 0 && aligned16(q) && aligned16(k) && aligned16(cos) &&
+                   aligned16(sin) && aligned16(q_out) && aligned16(k_out);
+  for (int64_t sd : strides) vector_ok = vector_ok && sd % vec == 0;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)num_tokens), block(256);
+  if (!vector_ok) {  // any even head size, any strides: one element pair per thread and step
+#define DLB_LAUNCH_ROTARY_ANY(DT_)                                                               \
+  hipLaunchKernelGGL(rotary_any_kernel<DT_>, grid, block, 0, s, q, k, cos, sin, q_out, k_out, Hq, \
+                     Hk, D, q_stride_tok, q_stride_head, k_stride_tok, k_stride_head,            \
+                     qo_stride_tok, qo_stride_head, ko_stride_tok, ko_stride_head, cs_stride_tok)
+    if (dtype == DLB_DTYPE_F32) DLB_LAUNCH_ROTARY_ANY(DLB_DTYPE_F32);
+    else if (dtype == DLB_DTYPE_BF16) DLB_LAUNCH_ROTARY_ANY(DLB_DTYPE_BF16);
+    else DLB_LAUNCH_ROTARY_ANY(DLB_DTYPE_F16);
+#undef DLB_LAUNCH_ROTARY_ANY
+    return launch_status();
+  }
   if (dtype == DLB_DTYPE_F32)
     hipLaunchKernelGGL(rotary_f32_kernel, grid, block, 0, s, (const float*)q, (const float*)k,
                        (const float*)cos, (const float*)sin, (float*)q_out, (float*)k_out, Hq, Hk,

@@ -6,8 +6,8 @@
 // points the reference leaves open fixed here: selection runs on the logits (the softmax is
 // monotone, so this is the same order without depending on exp rounding) and equal logits
 // resolve to the lowest expert index.  The fused softmax + K x argmax structure is that of
-// python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:24-60, minus its [K, S, E] int64
-// one-hot masks: indices are written directly.
+// python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:24-60; indices are written directly, and
+// that kernel's own outputs (the full softmax and the [K, S, E] int64 one-hot masks) on request.
 //
 // Mapping: a token is owned by one DPP row (16 lanes); every lane holds VPL consecutive
 // experts (VPL = 4 covers E <= 64 with one 128-bit load per lane), so a wave processes four
@@ -64,10 +64,15 @@ __device__ __forceinline__ void load_token_logits(const float* __restrict__ logi
 
 // Routes one token, whose logits the calling DPP row holds: lane r < K of the row stores the
 // r-th selected probability and expert and gets that expert back (other lanes and dead rows: -1).
+// probs / masks (either may be null) are the outputs in the form of the reference's fused gate
+// kernel (python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:47-60): the full softmax row
+// gates[token, :] and, for every selection round r, the one-hot row masks[r, token, :] (int64).
 template <int VPL>
 __device__ __forceinline__ int32_t route_token(const float (&v)[VPL], float* __restrict__ weights,
                                                int32_t* __restrict__ ids, int64_t token, bool live,
-                                               int E, int K, int renorm) {
+                                               int E, int K, int renorm,
+                                               float* __restrict__ probs = nullptr,
+                                               int64_t* __restrict__ masks = nullptr, int64_t T = 0) {
   const int lane16 = threadIdx.x & 15;
   const int e0 = lane16 * VPL;
 
@@ -84,6 +89,11 @@ __device__ __forceinline__ int32_t route_token(const float (&v)[VPL], float* __r
     sum += ex[j];
   }
   sum = row16_sum(sum);
+  if (probs && live) {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+      if (e0 + j < E) probs[token * E + e0 + j] = ex[j] / sum;  // the value a selected expert's weight has
+  }
 
   // K rounds of arg-max over (orderable(logit), 256 - index): ties -> lowest index.
   // tag 0 means "no candidate"; real candidates carry tag = 256 - index >= 1.
@@ -113,6 +123,11 @@ __device__ __forceinline__ int32_t route_token(const float (&v)[VPL], float* __r
     row_step_max<kDppRowHalfMirror>(bk, bt);
     row_step_max<kDppRowMirror>(bk, bt);
     const int sel = 256 - (int)bt;  // winning expert, identical on all 16 lanes
+    if (masks && live) {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j)
+        if (e0 + j < E) masks[((int64_t)r * T + token) * E + e0 + j] = (e0 + j == sel) ? 1 : 0;
+    }
     float p = 0.0f;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
@@ -142,11 +157,12 @@ __device__ __forceinline__ int32_t route_token(const float (&v)[VPL], float* __r
 template <int VPL>
 __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
     const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
-    int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok) {
+    int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok, float* __restrict__ probs,
+    int64_t* __restrict__ masks) {
   const int64_t token = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   float v[VPL];
   load_token_logits<VPL>(logits, token, token < T, E, ld, vec_ok, v);
-  route_token<VPL>(v, weights, ids, token, token < T, E, K, renorm);
+  route_token<VPL>(v, weights, ids, token, token < T, E, K, renorm, probs, masks, T);
 }
 
 // The router fused with the first step of the expert alignment: a workgroup of 1024 threads
@@ -210,8 +226,8 @@ int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids,
 }  // namespace dlb
 
 extern "C" int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids,
-                                        int64_t T, int E, int K, int64_t ld_logits,
-                                        int renormalize, void* stream) {
+                                        float* probs, int64_t* masks, int64_t T, int E, int K,
+                                        int64_t ld_logits, int renormalize, void* stream) {
   using namespace dlb;
   if (T < 0 || E < 1 || K < 1 || K > E || ld_logits < E) return DLB_ERR_BAD_ARG;
   if (K > 16 || E > 256) return DLB_ERR_UNSUPPORTED;
@@ -222,13 +238,13 @@ extern "C" int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int
   const bool a16 = aligned16(logits) && (ld_logits % 4 == 0);
   if (E <= 64) {
     hipLaunchKernelGGL(moe_topk_softmax_kernel<4>, grid, block, 0, s, logits, weights, ids, T, E,
-                       K, ld_logits, renormalize, (int)(a16 && E == 64));
+                       K, ld_logits, renormalize, (int)(a16 && E == 64), probs, masks);
   } else if (E <= 128) {
     hipLaunchKernelGGL(moe_topk_softmax_kernel<8>, grid, block, 0, s, logits, weights, ids, T, E,
-                       K, ld_logits, renormalize, (int)(a16 && E == 128));
+                       K, ld_logits, renormalize, (int)(a16 && E == 128), probs, masks);
   } else {
     hipLaunchKernelGGL(moe_topk_softmax_kernel<16>, grid, block, 0, s, logits, weights, ids, T, E,
-                       K, ld_logits, renormalize, (int)(a16 && E == 256));
+                       K, ld_logits, renormalize, (int)(a16 && E == 256), probs, masks);
   }
   return launch_status();
 }

@@ -12,11 +12,15 @@ import torch
 from .. import _lib
 
 
-def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True):
+def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True,
+                     return_probs: bool = False, return_masks: bool = False):
     """softmax(logits, fp32) -> top-k -> (optionally) weights / weights.sum(-1).
 
     Returns ``(weights fp32 [T, k], ids int32 [T, k])`` ordered by descending logit, equal
-    logits resolving to the lowest expert index.
+    logits resolving to the lowest expert index; with ``return_probs`` also the full softmax
+    ``probs fp32 [T, E]`` and with ``return_masks`` the one-hot selection rows
+    ``masks int64 [k, T, E]`` (the outputs of the reference's fused gate kernel,
+    python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:63-81), written by the same kernel.
     """
     assert logits.dim() == 2
     _lib.require_cuda(logits)
@@ -29,16 +33,25 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True):
         logits = logits.contiguous()
     weights = torch.empty((T, k), dtype=torch.float32, device=logits.device)
     ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    probs = torch.empty((T, E), dtype=torch.float32, device=logits.device) if return_probs else None
+    masks = torch.empty((k, T, E), dtype=torch.int64, device=logits.device) if return_masks else None
     if T > 0:
         lib = _lib.load()
         with _lib.device_guard(logits.device):
             st = lib.dlb_moe_topk_softmax_f32(logits.data_ptr(), weights.data_ptr(),
-                                              ids.data_ptr(), T, E, k,
+                                              ids.data_ptr(),
+                                              probs.data_ptr() if return_probs else None,
+                                              masks.data_ptr() if return_masks else None, T, E, k,
                                               logits.stride(0) if T > 1 else E,
                                               int(bool(renormalize)),
                                               _lib.current_stream_ptr(logits.device))
         _lib.check(st, "dlb_moe_topk_softmax_f32")
-    return weights, ids
+    out = (weights, ids)
+    if return_probs:
+        out += (probs,)
+    if return_masks:
+        out += (masks,)
+    return out
 
 
 def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int,

@@ -69,9 +69,15 @@ int dlb_silu_and_mul(const void* x, void* out, int64_t M, int64_t N, int64_t ld_
  * Selection is on the logits, descending, ties to the LOWEST expert index; weights are
  * p = exp(l - max) / sum(exp(l - max)) of the selected experts, divided by their sum when
  * renormalize != 0.  1 <= K <= 16, K <= E <= 256.
+ * Two optional outputs (NULL to skip) are those of the reference's fused gate kernel
+ * _topk_gating_kernel_part1 / call, kernels/topk_gating_fwd_part1.py:24-81:
+ *   probs fp32 [T, E] (contiguous): the full softmax row ("gates");
+ *   masks int64 [K, T, E] (contiguous): masks[r, t, :] is the one-hot row of the r-th selected
+ *         expert of token t (the reference's K rounds of argmax / overwrite, :52-60).
  * ---------------------------------------------------------------------------------------- */
-int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids, int64_t T,
-                             int E, int K, int64_t ld_logits, int renormalize, void* stream);
+int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids, float* probs,
+                             int64_t* masks, int64_t T, int E, int K, int64_t ld_logits,
+                             int renormalize, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * moe_align_block_size: per-expert counts, expert-sorted flat slot ids padded per expert to a
@@ -341,16 +347,20 @@ int dlb_fill_kv_cache(const void* k_states, const void* v_states, void* k_cache,
 /* rms_norm: out = weight * round(x * rsqrt(mean(x^2) + eps)); with `residual` != NULL the
  * input is first replaced by round(x + residual), which is also written to out_residual.
  * Replaces rms_norm / add_rms_norm, kernels/rms_norm.py:8-133 and kernels/add_rms_norm.py:9-80.
- * x/out/residual/out_residual [M, N] with row strides, weight [N]; bf16/f16 (N % 8 == 0) or
- * f32 (N % 4 == 0; nothing is rounded on the way), N <= 16384, 16-byte aligned rows. */
+ * x/out/residual/out_residual [M, N] with row strides, weight [N]; bf16/f16 or f32 (nothing is
+ * rounded on the way).  Any N >= 1: rows of whole 16-byte vectors (N % 8 == 0, f32 N % 4 == 0) up
+ * to 16384 elements with 16-byte aligned pointers and strides stay in registers between the sum of
+ * squares and the scaling; every other row length or alignment runs an element-wise kernel that
+ * reads the row twice (the reference masks the tail, kernels/rms_norm.py:8-75). */
 int dlb_rms_norm(const void* x, const void* weight, const void* residual, void* out,
                  void* out_residual, int64_t M, int N, int64_t ld_x, int64_t ld_res,
                  int64_t ld_out, int64_t ld_out_res, float eps, int dtype, void* stream);
 
 /* apply_rotary_pos_emb: out = x * cos + rotate_half(x) * sin on q [T, Hq, D] and k [T, Hk, D],
  * cos/sin [T, D] (row stride cs_stride_tok); outputs may alias the inputs.
- * Replaces apply_rotary_pos_emb, kernels/apply_rotary_pos_emb.py:8-164.  bf16/f16 (D % 16 == 0)
- * or f32 (D % 8 == 0); strides multiples of a 16-byte vector. */
+ * Replaces apply_rotary_pos_emb, kernels/apply_rotary_pos_emb.py:8-164.  bf16/f16/f32, any even
+ * D; 16-byte vectors are moved when D % 16 == 0 (f32: D % 8 == 0) and pointers and strides are
+ * multiples of a 16-byte vector, single elements otherwise. */
 int dlb_apply_rotary_pos_emb(const void* q, const void* k, const void* cos, const void* sin,
                              void* q_out, void* k_out, int64_t num_tokens, int Hq, int Hk, int D,
                              int64_t q_stride_tok, int64_t q_stride_head, int64_t k_stride_tok,

@@ -34,6 +34,26 @@ def topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True):
     return w, order.to(torch.int32)
 
 
+def topk_gating_part1(logits: torch.Tensor, k: int):
+    """``(gates [S, E], masks int64 [k, S, E])`` of the reference's fused gate kernel,
+    python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:47-60: ``gates = exp(x) / sum(exp(x))``
+    with the un-shifted exponential of the reference (:47-49), then k rounds of (arg-max, one-hot
+    row, overwrite the winner with ``finfo.min``) (:52-60).  The reference's ``tl.argmax`` leaves
+    the choice between equal values open; here it is the lowest index (``torch.argmax``)."""
+    x = logits.float()
+    ex = torch.exp(x)
+    gates = ex / ex.sum(dim=1, keepdim=True)
+    work = gates.clone()
+    fill = torch.finfo(torch.float32).min
+    masks = torch.zeros((k,) + tuple(gates.shape), dtype=torch.int64)
+    rows = torch.arange(gates.shape[0])
+    for i in range(k):
+        idx = work.argmax(dim=1)
+        masks[i, rows, idx] = 1
+        work[rows, idx] = fill
+    return gates.to(logits.dtype), masks
+
+
 def expert_counts(topk_ids: torch.Tensor, num_experts: int) -> torch.Tensor:
     flat = topk_ids.reshape(-1).long()
     flat = flat[(flat >= 0) & (flat < num_experts)]

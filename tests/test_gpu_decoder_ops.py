@@ -60,10 +60,9 @@ def test_fill_kv_cache_odd_head_dims_and_views(dev):
 
 # test_rms_norm.py:33-35: bf16, fp16 and fp32 on a (4, 8) input
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(4, 8), (3, 7, 4096), (64, 2048), (5, 11008), (2, 16384), (6, 12)])
+@pytest.mark.parametrize("shape", [(4, 8), (3, 7, 4096), (64, 2048), (5, 11008), (2, 16384), (6, 12),
+                                   (3, 1), (7, 77), (2, 16392), (2, 20000), (3, 4099)])
 def test_rms_norm(dev, dtype, shape):
-    if shape[-1] % 8 != 0 and dtype != torch.float32:
-        pytest.skip("16-bit rows are handled in 8-element vectors")
     from dlcompiler_amd.kernels.rms_norm import add_rms_norm, rms_norm
 
     g = torch.Generator().manual_seed(2)
@@ -90,7 +89,8 @@ def test_rms_norm(dev, dtype, shape):
 
 # test_apply_rotary.py:71-90: heads (8,8)/(8,4), feature dim 16, bf16/fp16/fp32, random positions
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("hq,hk,d", [(8, 8, 16), (8, 4, 16), (32, 8, 128), (5, 1, 64)])
+@pytest.mark.parametrize("hq,hk,d", [(8, 8, 16), (8, 4, 16), (32, 8, 128), (5, 1, 64), (3, 2, 2),
+                                     (4, 4, 6), (8, 2, 40), (2, 1, 100)])
 def test_apply_rotary(dev, dtype, hq, hk, d):
     from dlcompiler_amd.kernels.apply_rotary_pos_emb import apply_rotary_pos_emb
 

@@ -219,3 +219,60 @@ def test_output_width_comes_from_w2(dev, out_size):
     out = fused_moe_fp8(*[t.to(dev) for t in (x, w1q, w1s, w2q, w2s, tw, ids)], k)
     assert out.shape == (T, out_size)
     _check(out.cpu(), ref)
+
+
+# The GEMM keeps its accumulators relative to the scale of the current 128-deep chunk and moves
+# them from chunk to chunk with the ratio of neighbouring scales: rows whose neighbouring groups
+# differ by many orders of magnitude are the cases in which that ratio is extreme.  Every case is
+# checked against the dequantised fp32 evaluation at the usual tolerance and must stay finite.
+@pytest.mark.parametrize("case", ["zero_groups", "outlier_group", "tiny_activations",
+                                  "block_scale_spread", "scale_floor", "zero_weight_blocks"])
+def test_dynamic_range(dev, case):
+    from dlcompiler_amd.kernels import fused_moe as fm
+
+    T, H, I, E, k = 192, 1024, 512, 4, 2
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn((T, H), generator=g)
+    w1 = torch.randn((E, 2 * I, H), generator=g) * 0.05
+    w2 = torch.randn((E, H, I), generator=g) * 0.05
+    tw, ids = og.topk_softmax(torch.randn((T, E), generator=g), k, renormalize=True)
+    if case == "zero_groups":            # all-zero 128-groups between normal ones, and a zero row
+        x[::2, 128:256] = 0
+        x[::3, 512:768] = 0
+        x[1::4, 896:] = 0                # zero tail: the LAST chunk's scale is the eps scale
+        x[5] = 0
+    elif case == "outlier_group":        # one group 3000 x larger than its neighbours
+        x[:, 256:384] *= 3000.0
+        x[7, 0:128] *= 1e-4
+    elif case == "tiny_activations":     # an intermediate below the quantiser's eps (1e-10): its
+        x *= 1e-5                        # groups all carry the floor scale; some input groups too
+        x[::2, 384:512] *= 1e-7
+    x = x.to(torch.bfloat16)
+    w1q, w1s = ofp8.block_quant_weight(w1)
+    w2q, w2s = ofp8.block_quant_weight(w2)
+    if case == "block_scale_spread":     # block scales from 1e-6 to 1e+2 inside one expert
+        f = 10.0 ** torch.linspace(-6, 2, w1s[0].numel()).reshape(w1s[0].shape)
+        w1s = w1s * f[None] * 1e-3 / w1s.mean()
+        f2 = 10.0 ** torch.linspace(2, -6, w2s[0].numel()).reshape(w2s[0].shape)
+        w2s = w2s * f2[None] * 1e-3 / w2s.mean()
+    elif case == "scale_floor":          # block scales far below anything the kernel keeps apart
+        w1s[:, :, 2] = 1e-30
+        w1s[:, 1, :] = 1e-30
+        w2s[:, :, 1] = 1e-30
+    elif case == "zero_weight_blocks":   # all-zero weight blocks quantised with the scale 0
+        w1q8 = w1q.view(torch.uint8)
+        w1q8[:, 128:256, 256:384] = 0
+        w1q8[:, :, 896:] = 0             # the last chunk of every row
+        w1s[:, 1, 2] = 0.0
+        w1s[:, :, 7] = 0.0
+        w2q.view(torch.uint8)[:, 256:384, :128] = 0
+        w2s[:, 2, 0] = 0.0
+    ref = ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids)
+    assert torch.isfinite(ref.float()).all()
+    d = [t.to(dev) for t in (x, w1q, w1s, w2q, w2s, tw, ids)]
+    for shuffled in (False, True):
+        if shuffled:
+            d[1], d[3] = fm.shuffle_moe_weight_fp8(d[1]), fm.shuffle_moe_weight_fp8(d[3])
+        out = fm.fused_moe_fp8(*d, k, weights_shuffled=shuffled).cpu()
+        assert torch.isfinite(out.float()).all()
+        assert _rel_err(out, ref) <= 3e-2, (case, _rel_err(out, ref))

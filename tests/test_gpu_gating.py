@@ -30,6 +30,39 @@ def test_topk_softmax_parity(dev, T, E, k, renorm):
     torch.testing.assert_close(w, rw, rtol=1e-6, atol=0)        # north-star: 1e-6 relative
 
 
+# the reference's fused gate kernel in its own output form (topk_gating_fwd_part1.py:63-81):
+# full softmax gates [S, E] and one-hot masks [k, S, E] int64
+@pytest.mark.parametrize("S,E,k,dtype", [(16384, 64, 6, torch.float32), (4096, 64, 8, torch.float32),
+                                         (333, 60, 6, torch.float32), (50, 160, 6, torch.float32),
+                                         (19, 256, 16, torch.float32), (5, 3, 3, torch.float32),
+                                         (777, 64, 2, torch.float16)])
+def test_topk_gating_part1_outputs(dev, S, E, k, dtype):
+    from dlcompiler_amd.kernels.moe_gating import moe_topk_softmax
+    from dlcompiler_amd.kernels.topk_gating_fwd_part1 import call
+
+    g = torch.Generator().manual_seed(S + E)
+    logits = torch.randn((S, E), generator=g).to(dtype)
+    gates, masks = call(logits.to(dev), k)
+    assert gates.shape == (S, E) and gates.dtype == dtype
+    assert masks.shape == (k, S, E) and masks.dtype == torch.int64
+    rg, rm = og.topk_gating_part1(logits, k)
+    tol = dict(rtol=2e-6, atol=0) if dtype == torch.float32 else dict(rtol=2e-3, atol=1e-7)
+    torch.testing.assert_close(gates.cpu(), rg, **tol)
+    # the selection is unique where the top-(k+1) gate values of the oracle are distinct (it
+    # selects on rounded probabilities, the kernel on the logits)
+    top = torch.topk(rg.float(), min(k + 1, E), dim=-1).values
+    unique = (top[:, :-1] != top[:, 1:]).all(-1)
+    assert unique.float().mean() > 0.95
+    m = masks.cpu()
+    assert torch.equal(m[:, unique], rm[:, unique])
+    assert (m.sum(-1) == 1).all() and (m.sum(0) <= 1).all()
+    # the index form and the one-hot form come from one kernel and say the same
+    w, ids = moe_topk_softmax(logits.to(dev), k, renormalize=False)
+    assert torch.equal(m.argmax(-1).t().to(torch.int32), ids.cpu())
+    assert torch.equal(torch.gather(gates.float().cpu(), 1, ids.cpu().long()),
+                       w.cpu()) or dtype != torch.float32
+
+
 def test_topk_ties_resolve_to_lowest_index(dev):
     logits = torch.zeros((40, 64))
     logits[1, 10:20] = 2.0

@@ -124,3 +124,37 @@ def test_align_drops_out_of_range_ids():
     s, e, tot, cnt = og.align_block_size(ids, 2, 2)
     assert cnt.tolist() == [1, 2] and tot.item() == 4
     assert s.tolist()[:4] == [0, 6, 3, 5]
+
+
+def test_part1_is_softmax_plus_k_rounds_of_argmax():
+    # topk_gating_fwd_part1.py:47-60 against the library routines it is made of
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn((2048, 64), generator=g)
+    k = 6
+    gates, masks = og.topk_gating_part1(logits, k)
+    assert gates.shape == (2048, 64) and masks.shape == (k, 2048, 64) and masks.dtype == torch.int64
+    p = torch.softmax(logits, dim=-1)
+    torch.testing.assert_close(gates, p, rtol=2e-6, atol=0)      # un-shifted vs shifted exponent
+    assert (masks.sum(-1) == 1).all()                             # one expert per round
+    assert (masks.sum(0) <= 1).all()                              # never the same expert twice
+    # rows whose top-(k+1) softmax values are distinct have a unique answer: torch.topk's
+    top = torch.topk(p, k + 1, dim=-1)
+    unique = (top.values[:, :-1] != top.values[:, 1:]).all(-1)
+    gt = torch.topk(gates, k + 1, dim=-1).values
+    unique &= (gt[:, :-1] != gt[:, 1:]).all(-1)
+    assert unique.float().mean() > 0.99
+    picked = masks.argmax(-1).t()                                 # [S, k]
+    assert torch.equal(picked[unique], top.indices[unique][:, :k])
+    # and the index form of the router says the same
+    _, ids = og.topk_softmax(logits, k)
+    assert torch.equal(picked[unique], ids[unique].long())
+
+
+def test_part1_crafted_ties_and_fp16():
+    logits = torch.tensor([[1.0, 3.0, 3.0, -2.0, 3.0, 0.5, 0.5, 1.0],
+                           [0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0]])
+    gates, masks = og.topk_gating_part1(logits, 4)
+    assert masks.argmax(-1).t().tolist() == [[1, 2, 4, 0], [0, 1, 2, 3]]   # lowest index first
+    torch.testing.assert_close(gates.sum(-1), torch.ones(2))
+    g16, m16 = og.topk_gating_part1(logits.half(), 4)
+    assert g16.dtype == torch.float16 and torch.equal(m16, masks)
