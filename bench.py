@@ -151,6 +151,26 @@ def _cpu_info(cores=None):
             "cpu_model": _cpu_model(), "cpu_count": os.cpu_count()}
 
 
+def _cpu_time(fn, reps=3, warm=None):
+    """Seconds per call of a CPU-oracle leg: one untimed warm-up call (``warm`` if given, a cheaper
+    call that touches the same code paths, else ``fn`` itself), then the median of ``reps`` timed
+    calls."""
+    (warm or fn)()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+TRAFFIC_NOTE = ("traffic = bytes that missed the L2 per launch (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, "
+                "scaled by a copy kernel of known size), read from profiles/hbm_traffic.json -- a separate, "
+                "committed run, not this one; hits in the 256 MB Infinity Cache are inside it, so it is an "
+                "upper bound of the HBM bytes")
+
+
 def _traffic(name):
     """HBM bytes per launch of the named kernel from the committed rocprofv3 --pmc summary (a
     separate run: counters cannot be read inside this process), or None."""
@@ -193,15 +213,10 @@ def wl_silu(dev, steps, warmup, cpu):
 
         rows = 1024
         sample = x0[:rows]
-        oa.silu_and_mul(sample[:64])
-        t0 = time.perf_counter()
-        reps = 3
-        for _ in range(reps):
-            oa.silu_and_mul(sample)
-        dt = (time.perf_counter() - t0) / reps
+        dt = _cpu_time(lambda: oa.silu_and_mul(sample), warm=lambda: oa.silu_and_mul(sample[:64]))
         res["cpu_baseline"] = {"value": bytes_ * rows / M / dt / 1e9, "unit": "GB/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": f"{rows} of {M} rows, {reps} reps"}
+                               "sample": f"{rows} of {M} rows, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -283,15 +298,14 @@ def wl_gating(dev, steps, warmup, cpu):
     if cpu:
         from oracle import moe_gating as og
 
-        t0 = time.perf_counter()
-        reps = 3
-        for _ in range(reps):
+        def cpu_step():
             w, ids = og.topk_softmax(logits_cpu, K)
             og.align_block_size(ids, BLK, E)
-        dt = (time.perf_counter() - t0) / reps
+
+        dt = _cpu_time(cpu_step)
         res["cpu_baseline"] = {"value": bytes_ / dt / 1e9, "unit": "GB/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": f"full workload, {reps} reps"}
+                               "sample": "full workload, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -331,13 +345,11 @@ def wl_prefill(dev, steps, warmup, cpu):
 
         L = 1024  # one 1024-token sequence, all heads
         qs, ks, vs = q_cpu[:L], k_cpu[:L], v_cpu[:L]
-        t0 = time.perf_counter()
-        oa.prefill_attention(qs, ks, vs, torch.tensor([0]), torch.tensor([L]))
-        dt = time.perf_counter() - t0
+        dt = _cpu_time(lambda: oa.prefill_attention(qs, ks, vs, torch.tensor([0]), torch.tensor([L])))
         sflops = 4 * 128 * 32 * L * (L + 1) // 2
         res["cpu_baseline"] = {"value": sflops / dt / 1e12, "unit": "TFLOP/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": f"one {L}-token sequence, 32 heads, 1 rep"}
+                               "sample": f"one {L}-token sequence, 32 heads, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -388,13 +400,12 @@ def wl_decode(dev, steps, warmup, cpu):
         from oracle import attention as oa
 
         n = 8
-        t0 = time.perf_counter()
-        oa.paged_decode(q_cpu[:n], kc_cpu, vc_cpu, table[:n], ctx[:n])
-        dt = time.perf_counter() - t0
+        dt = _cpu_time(lambda: oa.paged_decode(q_cpu[:n], kc_cpu, vc_cpu, table[:n], ctx[:n]),
+                       warm=lambda: oa.paged_decode(q_cpu[:1], kc_cpu, vc_cpu, table[:1], ctx[:1]))
         sbytes = int(ctx[:n].sum()) * HKV * D * 4
         res["cpu_baseline"] = {"value": sbytes / dt / 1e9, "unit": "GB/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": f"first {n} of {B} sequences, 1 rep"}
+                               "sample": f"first {n} of {B} sequences, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -537,13 +548,11 @@ def wl_add_rms_norm(dev, steps, warmup, cpu):
     if cpu:
         from oracle import decoder_ops as od
 
-        x, r = xs[0][:2048].cpu(), rs[0][:2048].cpu()
-        t0 = time.perf_counter()
-        od.rms_norm(x, w.cpu(), 1e-6, residual=r)
-        dt = time.perf_counter() - t0
+        x, r, wc = xs[0][:2048].cpu(), rs[0][:2048].cpu(), w.cpu()
+        dt = _cpu_time(lambda: od.rms_norm(x, wc, 1e-6, residual=r))
         res["cpu_baseline"] = {"value": bytes_ * 2048 / M / dt / 1e9, "unit": "GB/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": f"2048 of {M} rows, 1 rep"}
+                               "sample": f"2048 of {M} rows, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -570,12 +579,11 @@ def wl_rotary(dev, steps, warmup, cpu):
         from oracle import decoder_ops as od
 
         n = 2048
-        t0 = time.perf_counter()
-        od.apply_rotary_pos_emb(qs[0][:n].cpu(), ks[0][:n].cpu(), cos[:n, None].cpu(), sin[:n, None].cpu())
-        dt = time.perf_counter() - t0
+        cq, ck, cc, cs_ = qs[0][:n].cpu(), ks[0][:n].cpu(), cos[:n, None].cpu(), sin[:n, None].cpu()
+        dt = _cpu_time(lambda: od.apply_rotary_pos_emb(cq, ck, cc, cs_))
         res["cpu_baseline"] = {"value": bytes_ * n / T / dt / 1e9, "unit": "GB/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": f"{n} of {T} tokens, 1 rep"}
+                               "sample": f"{n} of {T} tokens, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -613,13 +621,13 @@ def wl_fill_kv_cache(dev, steps, warmup, cpu):
     if cpu:
         from oracle import decoder_ops as od
 
-        t0 = time.perf_counter()
-        od.fill_kv_cache(k[0][:int(lens[0])].cpu(), v[0][:int(lens[0])].cpu(), kc[0].cpu(), vc[0].cpu(),
-                         [int(lens[0])], [0], table[:1])
-        dt = time.perf_counter() - t0
-        res["cpu_baseline"] = {"value": bytes_ * int(lens[0]) / T / dt / 1e9, "unit": "GB/s",
+        l0 = int(lens[0])
+        ck, cv, ckc, cvc = k[0][:l0].cpu(), v[0][:l0].cpu(), kc[0].cpu(), vc[0].cpu()
+        dt = _cpu_time(lambda: od.fill_kv_cache(ck, cv, ckc, cvc, [l0], [0], table[:1]))
+        res["cpu_baseline"] = {"value": bytes_ * l0 / T / dt / 1e9, "unit": "GB/s",
                                **_cpu_info(1), "kind": "port",
-                               "sample": f"first sequence ({int(lens[0])} tokens), 1 rep (includes a copy of the cache)"}
+                               "sample": f"first sequence ({l0} tokens), 1 warm-up + median of 3 reps "
+                                         "(each includes the oracle's copy of the cache)"}
     return res
 
 
@@ -666,14 +674,13 @@ def wl_paged_prefill(dev, steps, warmup, cpu):
     if cpu:
         from oracle import attention as oa
 
-        t0 = time.perf_counter()
-        oa.paged_prefill(q[:QL].cpu(), kc.cpu(), vc.cpu(), table[:1], torch.tensor([0]),
-                         torch.tensor([QL]), kvl[:1])
-        dt = time.perf_counter() - t0
+        cq, ckc, cvc = q[:QL].cpu(), kc.cpu(), vc.cpu()
+        dt = _cpu_time(lambda: oa.paged_prefill(cq, ckc, cvc, table[:1], torch.tensor([0]),
+                                                torch.tensor([QL]), kvl[:1]))
         f1 = 4 * D * HQ * (QL * int(hist[0]) + QL * (QL + 1) // 2)
         res["cpu_baseline"] = {"value": f1 / dt / 1e12, "unit": "TFLOP/s",
                                **_cpu_info(), "kind": "port",
-                               "sample": "first sequence, 1 rep"}
+                               "sample": "first sequence, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -864,6 +871,7 @@ def main():
         "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
                  "cpu_model": _cpu_model()},
         "box": box,
+        "traffic_note": TRAFFIC_NOTE,
         "workloads": results,
     }
     print(json.dumps(line))
