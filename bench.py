@@ -4,8 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
 Runs the five BASELINE.json configurations (fused silu_and_mul, MoE gating + alignment,
-varlen causal prefill attention, paged decode attention, fp8 fused-MoE MLP) and four neighbouring
-decoder-layer operators (add + RMSNorm, rotary embedding, KV-cache fill, paged prefill) on synthetic,
+varlen causal prefill attention, paged decode attention, fp8 fused-MoE MLP), the reference's own
+bf16 fused_moe at the config-5 shape and four neighbouring decoder-layer operators (add + RMSNorm,
+rotary embedding, KV-cache fill, paged prefill) on synthetic,
 seeded inputs that are resident in HBM before the timed region, and prints ONE JSON line.
 A "step" is one call of an operator's public entry point on one batch.  The top-level
 `metric`/`value`/`roofline`/`cpu_baseline` describe the primary workload (--workload, default
@@ -385,9 +386,14 @@ def wl_decode(dev, steps, warmup, cpu):
 
     ms, st = _time_steps(step, steps, warmup)
     ms_kernel = st["median_ms"]
+    # the same step with the index tensors as lmdeploy hands them over (int64): read as they are
+    table64, ctx64 = table_d.long(), ctx_d.long()
+    ms64, _ = _time_steps(lambda i: paged_attention_fwd(q, kcs[i % nbuf], vcs[i % nbuf], o, table64,
+                                                        None, ones, ctx64, 1), steps, warmup)
     res = {
         "metric": "paged decode attention HBM GB/s", "unit": "GB/s", "value": bytes_ / ms / 1e6,
         "ms_per_step": ms, "timing": st, "dtype": "bf16", "tflops": flops / ms / 1e9,
+        "int64_index_tensors": {"ms_per_step": ms64, "value": bytes_ / ms64 / 1e6, "unit": "GB/s"},
         "config": {"workload": "paged_attention_fwd decode, batch 64, ctx U[512,8192] seed 3, "
                                "64-token pages, 32q/8kv heads, d128, bf16",
                    "sum_ctx": sum_ctx, "algorithmic_bytes": bytes_},
@@ -512,6 +518,95 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         res["cpu_baseline"] = {"value": flops / dt / 1e12, "unit": "TFLOP/s",
                                **_cpu_info(), "kind": "port",
                                "sample": f"all {T} tokens, {reps} reps ({dt * reps:.1f} s of CPU time)"}
+    return res
+
+
+def wl_moe_bf16(dev, steps, warmup, cpu):
+    """The reference's own fused_moe (python/dlBLAS/dlblas/kernels/fused_moe.py:296-376) at the
+    config-5 shape in bf16: 4096 tokens, hidden 2048, intermediate 1408, 64 experts, top-6."""
+    from dlcompiler_amd import _lib
+    from dlcompiler_amd.kernels import fused_moe as fm
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size
+    from oracle import moe_gating as og
+
+    T, H, I, E, K = 4096, 2048, 1408, 64, 6
+    g = _gen(5)
+    x_cpu = torch.randn((T, H), generator=g).bfloat16()
+    logits = torch.randn((T, E), generator=g)
+    tw_cpu, ids_cpu = og.topk_softmax(logits, K)   # input preparation, untimed
+    w1_cpu = torch.empty((E, 2 * I, H), dtype=torch.bfloat16)
+    w2_cpu = torch.empty((E, H, I), dtype=torch.bfloat16)
+    for e in range(E):
+        w1_cpu[e] = (torch.randn((2 * I, H), generator=g) * 0.02).bfloat16()
+        w2_cpu[e] = (torch.randn((H, I), generator=g) * 0.02).bfloat16()
+    x, tw, ids = x_cpu.to(dev), tw_cpu.to(dev), ids_cpu.to(dev)
+    plain = [w1_cpu.to(dev), w2_cpu.to(dev)]
+    shuf = [fm.shuffle_moe_weight(plain[0]), fm.shuffle_moe_weight(plain[1])]
+    gate_up_flops, down_flops = 2 * T * K * H * 2 * I, 2 * T * K * I * H
+    flops = gate_up_flops + down_flops
+
+    def kernel_times(dw, shuffled):
+        lib = _lib.load()
+        block = fm._BLOCK_M
+        sorted_ids, _, _, counts = moe_align_block_size(ids, block, E, return_counts=True)
+        nmb = sorted_ids.numel() // block
+        act = torch.empty((nmb * block, I), dtype=torch.bfloat16, device=dev)
+        slots = torch.empty((T * K, H), dtype=torch.bfloat16, device=dev)
+        stream = _lib.current_stream_ptr(dev)
+
+        def gate_up(i):
+            _lib.check(lib.dlb_moe_gemm_16bit_gate_up(
+                x.data_ptr(), dw[0].data_ptr(), sorted_ids.data_ptr(), counts.data_ptr(), E, nmb, block,
+                T, K, H, I, 0, E, int(shuffled), act.data_ptr(), 0, stream), "gate_up")
+
+        def down(i):
+            _lib.check(lib.dlb_moe_gemm_16bit_down(
+                act.data_ptr(), dw[1].data_ptr(), sorted_ids.data_ptr(), counts.data_ptr(), E,
+                tw.data_ptr(), nmb, block, T, K, H, I, 0, E, int(shuffled), slots.data_ptr(), 0,
+                stream), "down")
+
+        for i in range(MIN_WARMUP):
+            gate_up(i)
+            down(i)
+        return _batch_stats(gate_up), _batch_stats(down)
+
+    layouts = {}
+    for name, dw, shuffled in (("row-major", plain, False), ("operand-order", shuf, True)):
+        ms, st = _time_steps(lambda i: fm.fused_moe(x, *dw, tw, ids, K, weights_shuffled=shuffled),
+                             steps, warmup)
+        st_gu, st_dn = kernel_times(dw, shuffled)
+        layouts[name] = {
+            "ms_per_step": ms, "value": flops / ms / 1e9, "unit": "TFLOP/s", "timing": st,
+            "gate_up_kernel": dict(st_gu, tflops=gate_up_flops / st_gu["median_ms"] / 1e9,
+                                   frac=gate_up_flops / st_gu["median_ms"] / 1e9 / PEAK_BF16_TFLOPS),
+            "down_kernel": dict(st_dn, tflops=down_flops / st_dn["median_ms"] / 1e9,
+                                frac=down_flops / st_dn["median_ms"] / 1e9 / PEAK_BF16_TFLOPS),
+        }
+    # the reference's signature and weight layout are the figure of this workload
+    ref_l = layouts["row-major"]
+    ms = ref_l["ms_per_step"]
+    ms_gate_up = ref_l["gate_up_kernel"]["median_ms"]
+    res = {
+        "metric": "bf16 fused-MoE TFLOP/s", "unit": "TFLOP/s", "value": flops / ms / 1e9,
+        "ms_per_step": ms, "timing": ref_l["timing"], "dtype": "bf16",
+        "config": {"workload": "fused_moe T=4096 H=2048 I=1408 E=64 top-6, bf16 weights in the "
+                               "reference's row-major [E, N, K] layout, seed 5",
+                   "algorithmic_flops": flops},
+        "weight_layouts": layouts,
+        "roofline": {"kernel": "moe_gemm_kernel<gate_up, bf16>", "bound": "mfma",
+                     "achieved": gate_up_flops / ms_gate_up / 1e9, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": gate_up_flops / ms_gate_up / 1e9 / PEAK_BF16_TFLOPS,
+                     "traffic": _traffic("moe_gemm_bf16_gate_up")},
+    }
+    if cpu:
+        from oracle import fused_moe as ofm
+
+        n = 1024   # a quarter of the tokens against all experts
+        dt = _cpu_time(lambda: ofm.fused_moe(x_cpu[:n], w1_cpu, w2_cpu, tw_cpu[:n], ids_cpu[:n]),
+                       warm=lambda: ofm.fused_moe(x_cpu[:64], w1_cpu, w2_cpu, tw_cpu[:64], ids_cpu[:64]))
+        res["cpu_baseline"] = {"value": flops * n / T / dt / 1e12, "unit": "TFLOP/s",
+                               **_cpu_info(), "kind": "port",
+                               "sample": f"first {n} of {T} tokens, 1 warm-up + median of 3 reps"}
     return res
 
 
@@ -794,6 +889,8 @@ WORKLOADS = {
     "prefill_attention": wl_prefill,
     "paged_decode": wl_decode,
     "moe_fp8": wl_moe_fp8,
+    # the reference's own fused_moe (bf16) at the same shape
+    "moe_bf16": wl_moe_bf16,
     # the neighbours of the five configurations in a decoder layer
     "add_rms_norm": wl_add_rms_norm,
     "apply_rotary_pos_emb": wl_rotary,
