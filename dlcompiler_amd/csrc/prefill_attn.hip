@@ -97,7 +97,11 @@ struct Smem {
 // likewise) only produce output dims that are never stored.  The reference handles odd head
 // sizes by splitting them into power-of-two blocks with masked loads
 // (python/dlBLAS/dlblas/kernels/paged_attention.py:531-539).
-template <int DT, int D, bool PAGED, bool RAGGED>
+// PAGED: 0 = packed K/V; 1 = paged, every K/V row looks up its own page (any page size); 2 = paged
+// with pages that are whole multiples of the 64-key tile: a tile lies in one page, so its page
+// number is one wave-uniform look-up and the copies are addressed as in the packed layout (a
+// scalar base per tile plus constant lane offsets).
+template <int DT, int D, int PAGED, bool RAGGED>
 __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int KS = D / 16;  // MFMA k-steps over the head dim for S^T
   constexpr int MT = D / 32;  // 32-row tiles of O^T
@@ -223,7 +227,13 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   // paged layout: the page ids of the rows this lane copies are fetched one tile ahead of the
   // copy that needs them, so the block-table latency never sits in front of a tile's copies
   int pg_next[KINS];
+  int pg_tile = 0;  // PAGED == 2: the page of the next tile to stage (wave-uniform)
   auto fetch_pages = [&](int t0) {
+    if (PAGED == 2) {
+      const int key = min(t0, kv_total - 1);
+      pg_tile = bt[p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page)];
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < KINS; ++i) {
       const int key = min(t0 + (4 * i + wave) * KRPI + k_lrow, kv_total - 1);
@@ -256,10 +266,19 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
       kbase = uniform_ptr(kbytes + (tok0 + t0) * k_row_bytes);
       vbase = uniform_ptr(vbytes + (tok0 + t0) * v_row_bytes);
     }
+    if (PAGED == 2) {
+      // t0 is a multiple of the tile and the page a multiple of the tile: slot of the tile's
+      // first key inside its page (a tile whose first key lies past the context is never staged)
+      const int pi = p.page_shift >= 0 ? (t0 >> p.page_shift) : (t0 / p.page);
+      const int64_t pg = __builtin_amdgcn_readfirstlane(pg_tile);
+      const int64_t slot0 = t0 - pi * p.page;
+      kbase = uniform_ptr(kbytes + (pg * p.k_sp + slot0 * p.k_st) * 2);
+      vbase = uniform_ptr(vbytes + (pg * p.v_sp + slot0 * p.v_st) * 2);
+    }
 #pragma unroll
     for (int i = 0; i < KINS; ++i) {
       const int r = (4 * i + wave) * KRPI + k_lrow;  // key row inside the tile
-      if (PAGED) {
+      if (PAGED == 1) {
         int key = t0 + r;
         if (CLAMP) key = min(key, kv_total - 1);
         const int pi = p.page_shift >= 0 ? (key >> p.page_shift) : (key / p.page);
@@ -280,7 +299,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const Prefill
   auto issue_copy = [&](int n) {
     const int i = n >> 1;  // 1 KB slice 4*i + wave of the tile
     const unsigned int dst = stage_dst + (n & 1) * SM::kBytes + i * 4096;
-    if (PAGED) dma16_global_to_lds((n & 1) ? vsrc[i] : ksrc[i], dst);
+    if (PAGED == 1) dma16_global_to_lds((n & 1) ? vsrc[i] : ksrc[i], dst);
     else if (n & 1) dma16_global_to_lds(vbase, voff[i], dst);
     else dma16_global_to_lds(kbase, koff[i], dst);
   };
@@ -541,7 +560,11 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk,
     if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 128, PG_);  \
     else DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 64, PG_);            \
   }
-  if (paged) { DLB_DISPATCH_PREFILL(true) } else { DLB_DISPATCH_PREFILL(false) }
+  // pages that hold whole 64-key tiles take the kernel with one page look-up per tile (the lane
+  // offsets inside a page are 32-bit)
+  const bool tile_pages = paged && p.page % kTileN == 0 &&
+                          (int64_t)p.page * p.k_st * 2 <= 0x7fffffff && (int64_t)p.page * p.v_st * 2 <= 0x7fffffff;
+  if (tile_pages) { DLB_DISPATCH_PREFILL(2) } else if (paged) { DLB_DISPATCH_PREFILL(1) } else { DLB_DISPATCH_PREFILL(0) }
 #undef DLB_DISPATCH_PREFILL
 #undef DLB_LAUNCH_PREFILL
   return launch_status();
