@@ -29,6 +29,10 @@ SIGNATURES = {
     "dlb_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                          c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                          c_size_t, c_void_p]),
+    "dlb_moe_align_quant_fp8": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+                                        c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_size_t,
+                                        c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
+                                        c_int64, c_int64, c_int, c_void_p]),
     "dlb_moe_align_block_size_static_max_numel": (c_int64, []),
     "dlb_moe_align_block_size_static": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
                                                 c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),

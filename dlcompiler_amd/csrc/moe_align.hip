@@ -19,27 +19,42 @@
 #include <mutex>
 
 #include "common.h"
+#include "quant_fp8.h"
 
 namespace dlb {
 namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
-constexpr int kChunk = 2048;  // flat ids per workgroup
+constexpr int kChunk = 2048;  // flat ids per workgroup (large inputs)
 constexpr int kMaxE = 256;
+constexpr int kFusedChunks = 256;  // rows of the count table the fused placement kernel reduces
+static_assert(kFusedChunks == kRouteMaxChunks, "the fused router sizes its chunks for this table");
 
+// Flat ids per chunk (= per workgroup of the counting and the placement pass).  Inputs of up to
+// kFusedChunks * kChunk ids are cut into as many chunks as the fused placement kernel takes (256),
+// but not below one tile of 256 ids: a decoder layer's 25 k - 100 k routing slots then run on
+// 96 - 256 workgroups with one or two tiles each instead of 12 - 48 workgroups that walk eight
+// tiles one after the other.  Larger inputs use chunks of kChunk ids and the three-launch path.
+__host__ __device__ inline int chunk_ids_for(int64_t numel) {
+  if (numel > (int64_t)kFusedChunks * kChunk) return kChunk;
+  const int64_t per = (numel + kFusedChunks - 1) / kFusedChunks;
+  const int64_t rounded = (per + 63) / 64 * 64;
+  return (int)(rounded < kThreads ? kThreads : rounded);
+}
 __host__ __device__ inline int64_t num_chunks(int64_t numel) {
-  return numel > 0 ? (numel + kChunk - 1) / kChunk : 1;
+  const int c = chunk_ids_for(numel);
+  return numel > 0 ? (numel + c - 1) / c : 1;
 }
 
 __global__ __launch_bounds__(kThreads) void align_count_kernel(const int32_t* __restrict__ ids,
-                                                               int64_t numel, int E,
+                                                               int64_t numel, int E, int chunk_ids,
                                                                int32_t* __restrict__ chunk_counts) {
   __shared__ int32_t hist[kMaxE];
   for (int e = threadIdx.x; e < E; e += kThreads) hist[e] = 0;
   __syncthreads();
-  const int64_t begin = (int64_t)blockIdx.x * kChunk;
-  const int64_t end = begin + kChunk < numel ? begin + kChunk : numel;
+  const int64_t begin = (int64_t)blockIdx.x * chunk_ids;
+  const int64_t end = begin + chunk_ids < numel ? begin + chunk_ids : numel;
   for (int64_t i = begin + threadIdx.x; i < end; i += kThreads) {
     const int32_t e = ids[i];
     if (e >= 0 && e < E) atomicAdd(&hist[e], 1);  // integer add: order-insensitive
@@ -185,14 +200,31 @@ __global__ __launch_bounds__(kThreads) void align_place_kernel(
 // the offsets of its own chunk -- instead of waiting for a separate one-workgroup scan kernel;
 // one extra workgroup emits what the scan kernel emits (counts, block -> expert ids, pad slots,
 // tails, padded total).  The table is only read here.
-constexpr int kFusedChunks = 256;
-static_assert(kFusedChunks == kRouteMaxChunks, "the fused router sizes its chunks for this table");
+struct PlaceParams {
+  const int32_t* ids;
+  int64_t numel;
+  int E, block;
+  const int32_t* chunk_counts;
+  int chunks, chunk_ids;
+  int32_t* sorted_ids;
+  int64_t sorted_cap;
+  int32_t* expert_ids;
+  int64_t expert_ids_cap;
+  int32_t* counts;
+  int32_t* num_post_pad;
+};
 
-__global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
-    const int32_t* __restrict__ ids, int64_t numel, int E, int block,
-    const int32_t* __restrict__ chunk_counts, int chunks, int chunk_ids,
-    int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_ids_cap, int32_t* __restrict__ counts, int32_t* __restrict__ num_post_pad) {
+// the work of workgroup `me` (0 .. chunks) of the fused scan + placement
+__device__ __forceinline__ void align_place_fused_block(const PlaceParams& pp, const int me) {
+  const int32_t* __restrict__ ids = pp.ids;
+  const int64_t numel = pp.numel;
+  const int E = pp.E, block = pp.block, chunks = pp.chunks, chunk_ids = pp.chunk_ids;
+  const int32_t* __restrict__ chunk_counts = pp.chunk_counts;
+  int32_t* __restrict__ sorted_ids = pp.sorted_ids;
+  const int64_t sorted_cap = pp.sorted_cap, expert_ids_cap = pp.expert_ids_cap;
+  int32_t* __restrict__ expert_ids = pp.expert_ids;
+  int32_t* __restrict__ counts = pp.counts;
+  int32_t* __restrict__ num_post_pad = pp.num_post_pad;
   __shared__ int32_t cursor[kMaxE];            // next free slot per expert for this chunk
   __shared__ int32_t wave_cnt[kWaves][kMaxE];  // per-tile, per-wave counts
   __shared__ int32_t total_s[kMaxE];
@@ -200,7 +232,6 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid / kWave;
-  const int me = blockIdx.x;
 
   // this chunk's first ids are requested before the count table is reduced (they do not depend
   // on it), each later tile's while the tile before it is placed
@@ -228,11 +259,21 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
     const int c0 = q * per, c1 = min(c0 + per, chunks);
     int32_t total = 0, before_part = 0;
     if (e < E && q < groups) {
-#pragma unroll 8  // independent loads: eight rows in flight instead of one round trip each
-      for (int c = c0; c < c1; ++c) {
-        const int32_t n = chunk_counts[(int64_t)c * E + e];
-        total += n;
-        if (c < me) before_part += n;
+      // The table was written by the launch before this one, on other XCDs: every dependent batch
+      // of loads is a full memory round trip.  All rows of the slice are therefore requested at
+      // once (64 per thread cover 256 chunks of up to 64 experts; wider expert counts take a
+      // second or fourth batch).
+      constexpr int kRowsInFlight = 64;
+      for (int cb = c0; cb < c1; cb += kRowsInFlight) {
+        int32_t n[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u)
+          n[u] = (cb + u < c1) ? chunk_counts[(int64_t)(cb + u) * E + e] : 0;
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+          total += n[u];
+          if (cb + u < me) before_part += n[u];
+        }
       }
     }
     int32_t* part = &wave_cnt[0][0];  // [2][groups][ep] <= 2 * 256 entries
@@ -327,6 +368,22 @@ __global__ __launch_bounds__(kThreads) void align_place_fused_kernel(
   }
 }
 
+__global__ __launch_bounds__(kThreads) void align_place_fused_kernel(const PlaceParams pp) {
+  align_place_fused_block(pp, blockIdx.x);
+}
+
+// The fused scan + placement and the fp8 activation quantiser in ONE launch: workgroups
+// 0 .. chunks run the placement, the ones after them quantise.  The two jobs share nothing; run
+// side by side they cost one launch and the longer of the two instead of two launches.
+static_assert(kQuantThreads == kThreads, "one workgroup size for both jobs");
+template <int DT>
+__global__ __launch_bounds__(kThreads) void align_place_quant_kernel(const PlaceParams pp,
+                                                                     const QuantParams q) {
+  const int nplace = pp.chunks + 1;
+  if ((int)blockIdx.x < nplace) align_place_fused_block(pp, blockIdx.x);
+  else quant_fp8_group128_block<DT>(q, (int64_t)blockIdx.x - nplace);
+}
+
 }  // namespace
 }  // namespace dlb
 
@@ -356,17 +413,29 @@ int check_align_args(const int32_t* topk_ids, int64_t numel, int E, int block,
 // which the counting pass overwrites before anything reads it (nothing has to start at zero)
 int launch_align(const int32_t* topk_ids, int64_t numel, int E, int block, int32_t* sorted_ids,
                  int64_t sorted_cap, int32_t* expert_ids, int64_t expert_ids_cap, int32_t* counts,
-                 int32_t* num_post_pad, int32_t* chunk_counts, hipStream_t s) {
+                 int32_t* num_post_pad, int32_t* chunk_counts, hipStream_t s,
+                 const QuantParams* quant = nullptr, int quant_dtype = DLB_DTYPE_BF16) {
   const int64_t chunks = num_chunks(numel);
+  const int chunk_ids = chunk_ids_for(numel);
   hipLaunchKernelGGL(align_count_kernel, dim3((uint32_t)chunks), dim3(kThreads), 0, s, topk_ids,
-                     numel, E, chunk_counts);
+                     numel, E, chunk_ids, chunk_counts);
   if (chunks <= kFusedChunks) {
     // (with numel = 0 the single chunk is empty: the extra workgroup still writes pads, tails and totals)
-    hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s,
-                       topk_ids, numel, E, block, chunk_counts, (int)chunks, kChunk, sorted_ids,
-                       sorted_cap, expert_ids, expert_ids_cap, counts, num_post_pad);
+    const PlaceParams pp = {topk_ids,   numel,      E,          block,          chunk_counts, (int)chunks,
+                            chunk_ids,  sorted_ids, sorted_cap, expert_ids,     expert_ids_cap,
+                            counts,     num_post_pad};
+    if (quant && quant->total_groups > 0) {
+      const uint32_t grid = (uint32_t)(chunks + 1 + ceil_div(quant->total_groups, kQuantGroupsPerBlock));
+      if (quant_dtype == DLB_DTYPE_BF16)
+        hipLaunchKernelGGL(align_place_quant_kernel<DLB_DTYPE_BF16>, dim3(grid), dim3(kThreads), 0, s, pp, *quant);
+      else
+        hipLaunchKernelGGL(align_place_quant_kernel<DLB_DTYPE_F16>, dim3(grid), dim3(kThreads), 0, s, pp, *quant);
+    } else {
+      hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s, pp);
+    }
     return launch_status();
   }
+  if (quant) return DLB_ERR_UNSUPPORTED;  // (the caller launches the quantiser on its own then)
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, chunk_counts, chunks, E, block,
                      (int32_t)numel, sorted_ids, sorted_cap, expert_ids, expert_ids_cap, counts,
                      num_post_pad);
@@ -422,8 +491,34 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
                       expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream);
 }
 
+extern "C" int dlb_moe_align_quant_fp8(const int32_t* topk_ids, int64_t numel, int E, int block,
+                                       int32_t* sorted_ids, int64_t sorted_cap,
+                                       int32_t* expert_ids, int64_t expert_ids_cap,
+                                       int32_t* counts, int32_t* num_post_pad, void* ws,
+                                       size_t ws_bytes, const void* x, void* xq, float* xs,
+                                       int64_t M, int K, int64_t ld_x, int64_t ld_q, int64_t ld_s,
+                                       int dtype, void* stream) {
+  using namespace dlb;
+  const int st = check_align_args(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                                  expert_ids_cap, num_post_pad);
+  if (st != DLB_OK) return st;
+  if (!ws || ws_bytes < dlb_moe_align_ws_bytes(numel, E)) return DLB_ERR_WORKSPACE;
+  QuantParams q;
+  const int sq = fill_quant_params(q, x, xq, xs, M, K, ld_x, ld_q, ld_s, dtype);
+  if (sq != DLB_OK) return sq;
+  if (num_chunks(numel) <= kFusedChunks)
+    return launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                        expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream, &q,
+                        dtype);
+  // more routing slots than the fused placement takes: the separate launches
+  const int sa = launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+                              expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream);
+  if (sa != DLB_OK) return sa;
+  return dlb_per_token_group_quant_fp8(x, xq, xs, M, K, ld_x, ld_q, ld_s, dtype, stream);
+}
+
 extern "C" int64_t dlb_moe_align_block_size_static_max_numel(void) {
-  return (int64_t)dlb::kStaticChunks * dlb::kChunk;
+  return (int64_t)dlb::kStaticChunks * dlb::kChunk;  // = kFusedChunks chunks of the largest size
 }
 
 extern "C" int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int E,
@@ -484,10 +579,12 @@ extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weight
     if (st != DLB_OK) return st;
   } else {
     // no tokens: the single chunk is empty, but its row of the table is still read
-    hipLaunchKernelGGL(align_count_kernel, dim3(1), dim3(kThreads), 0, s, ids, (int64_t)0, E, chunk_counts);
+    hipLaunchKernelGGL(align_count_kernel, dim3(1), dim3(kThreads), 0, s, ids, (int64_t)0, E, kChunk,
+                       chunk_counts);
   }
-  hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s, ids,
-                     numel, E, block, chunk_counts, (int)chunks, chunk_tokens * K, sorted_ids,
-                     sorted_cap, expert_ids, expert_ids_cap, counts, num_post_pad);
+  const PlaceParams pp = {ids,        numel,      E,          block,          chunk_counts, (int)chunks,
+                          chunk_tokens * K, sorted_ids, sorted_cap, expert_ids, expert_ids_cap,
+                          counts,     num_post_pad};
+  hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s, pp);
   return launch_status();
 }

@@ -27,12 +27,11 @@
 #include <type_traits>
 
 #include "common.h"
+#include "quant_fp8.h"
 
 namespace dlb {
 namespace {
 
-constexpr float kFp8Max = 448.0f;
-constexpr float kQuantEps = 1e-10f;
 // K chunks of 128 bytes whose block scales the fp8 grouped GEMM parks in LDS: reduction lengths
 // up to 128 * 128 = 16384 (checked on the host before the launch)
 constexpr int kMoeMaxKChunks = 128;
@@ -45,61 +44,12 @@ constexpr int kMoeMaxKChunks = 128;
 constexpr float kActScaleFloor = 1e-13f;
 constexpr float kWScaleFloor = 1e-12f;
 
-__device__ __forceinline__ unsigned int pack4_fp8(float a, float b, float c, float d) {
-  // v_cvt_pk_fp8_f32 rounds to nearest even; values beyond +-464 would become NaN, so clamp.
-  a = fminf(fmaxf(a, -kFp8Max), kFp8Max);
-  b = fminf(fmaxf(b, -kFp8Max), kFp8Max);
-  c = fminf(fmaxf(c, -kFp8Max), kFp8Max);
-  d = fminf(fmaxf(d, -kFp8Max), kFp8Max);
-  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
-  return (unsigned int)r;
-}
-
 // ---------------------------------------------------------------------------------------
-// per-token-group quantisation: one DPP row (16 lanes x 8 elements) per 128-element group
+// per-token-group quantisation (the body lives in quant_fp8.h)
 // ---------------------------------------------------------------------------------------
-constexpr int kQuantUnroll = 4;  // groups per DPP row and workgroup pass (loads issued together)
-
 template <int DT>
-__global__ __launch_bounds__(256) void quant_fp8_group128_kernel(
-    const unsigned short* __restrict__ x, unsigned char* __restrict__ xq, float* __restrict__ xs,
-    int64_t total_groups, int groups_per_row, int64_t ldx, int64_t ldq, int64_t lds) {
-  const int lane16 = threadIdx.x & 15;
-  int64_t row[kQuantUnroll];
-  int gc[kQuantUnroll];
-  bool live[kQuantUnroll];
-  u32x4 raw[kQuantUnroll];
-#pragma unroll
-  for (int u = 0; u < kQuantUnroll; ++u) {
-    const int64_t gidx = ((int64_t)blockIdx.x * kQuantUnroll + u) * 16 + (threadIdx.x >> 4);
-    live[u] = gidx < total_groups;
-    row[u] = live[u] ? gidx / groups_per_row : 0;
-    gc[u] = live[u] ? (int)(gidx - row[u] * groups_per_row) : 0;
-    raw[u] = u32x4{0u, 0u, 0u, 0u};
-    if (live[u]) raw[u] = __builtin_nontemporal_load((const u32x4*)(x + row[u] * ldx + gc[u] * 128 + lane16 * 8));
-  }
-#pragma unroll
-  for (int u = 0; u < kQuantUnroll; ++u) {
-    float v[8];
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      v[2 * w] = Elem<DT>::lo(raw[u][w]);
-      v[2 * w + 1] = Elem<DT>::hi(raw[u][w]);
-    }
-    float amax = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
-    amax = row16_max(amax);
-    const float scale = fmaxf(amax, kQuantEps) / kFp8Max;
-    if (live[u]) {
-      u32x2 q;
-      q[0] = pack4_fp8(v[0] / scale, v[1] / scale, v[2] / scale, v[3] / scale);
-      q[1] = pack4_fp8(v[4] / scale, v[5] / scale, v[6] / scale, v[7] / scale);
-      *(u32x2*)(xq + row[u] * ldq + gc[u] * 128 + lane16 * 8) = q;
-      if (lane16 == 0) xs[row[u] * lds + gc[u]] = scale;
-    }
-  }
+__global__ __launch_bounds__(kQuantThreads) void quant_fp8_group128_kernel(const QuantParams q) {
+  quant_fp8_group128_block<DT>(q, blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -744,8 +694,11 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
   else run(std::integral_constant<int, 2>{});
 }
 
-// out[t, n] = sum_j in[t * topk + j, n], fp32 accumulation in slot order, one rounding
-template <int DT>
+// out[t, n] = sum_j in[t * topk + j, n], fp32 accumulation in slot order, one rounding.
+// TOPK > 0: the slot count is a compile-time constant and all its loads are requested before the
+// first is used (the kernel is a pure stream: what counts is the number of bytes in flight);
+// TOPK = 0: any slot count, four loads at a time.
+template <int DT, int TOPK>
 __global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restrict__ in,
                                                            u32x4* __restrict__ out,
                                                            int64_t total_vec, int vec_per_row,
@@ -757,18 +710,35 @@ __global__ __launch_bounds__(256) void moe_topk_sum_kernel(const u32x4* __restri
   float s[8];
 #pragma unroll
   for (int q = 0; q < 8; ++q) s[q] = 0.0f;
-  for (int j = 0; j < topk; ++j) {
-    const u32x4 v = __builtin_nontemporal_load(in + (t * topk + j) * vec_per_row + col);
+  auto add = [&](const u32x4& v) {
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       s[2 * w] += Elem<DT>::lo(v[w]);
       s[2 * w + 1] += Elem<DT>::hi(v[w]);
     }
+  };
+  const u32x4* row = in + t * (int64_t)(TOPK ? TOPK : topk) * vec_per_row + col;
+  if constexpr (TOPK > 0) {
+    u32x4 v[TOPK];
+#pragma unroll
+    for (int j = 0; j < TOPK; ++j) v[j] = __builtin_nontemporal_load(row + (int64_t)j * vec_per_row);
+#pragma unroll
+    for (int j = 0; j < TOPK; ++j) add(v[j]);
+  } else {
+    int j = 0;
+    for (; j + 4 <= topk; j += 4) {
+      u32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(row + (int64_t)(j + u) * vec_per_row);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) add(v[u]);
+    }
+    for (; j < topk; ++j) add(__builtin_nontemporal_load(row + (int64_t)j * vec_per_row));
   }
   u32x4 r;
 #pragma unroll
   for (int w = 0; w < 4; ++w) r[w] = Elem<DT>::pack(s[2 * w], s[2 * w + 1]);
-  out[i] = r;
+  __builtin_nontemporal_store(r, out + i);
 }
 
 }  // namespace
@@ -779,26 +749,16 @@ extern "C" int dlb_per_token_group_quant_fp8(const void* x, void* xq, float* xs,
                                              int K, int64_t ld_x, int64_t ld_q, int64_t ld_s,
                                              int dtype, void* stream) {
   using namespace dlb;
-  if (M < 0 || K < 0 || ld_x < K || ld_q < K || ld_s < K / 128) return DLB_ERR_BAD_ARG;
+  QuantParams q;
+  const int st = fill_quant_params(q, x, xq, xs, M, K, ld_x, ld_q, ld_s, dtype);
+  if (st != DLB_OK) return st;
   if (M == 0 || K == 0) return DLB_OK;
-  if (!x || !xq || !xs) return DLB_ERR_BAD_ARG;
-  if (K % 128 != 0 || ld_x % 8 != 0 || ld_q % 8 != 0 || !aligned16(x) ||
-      (reinterpret_cast<uintptr_t>(xq) & 7u) != 0)
-    return DLB_ERR_UNSUPPORTED;
-  const int gpr = K / 128;
-  const int64_t total = M * gpr;
-  const dim3 grid((uint32_t)ceil_div(total, 16 * kQuantUnroll));
+  const dim3 grid((uint32_t)ceil_div(q.total_groups, kQuantGroupsPerBlock));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DLB_DTYPE_BF16)
-    hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_BF16>, grid, dim3(256), 0, s,
-                       (const unsigned short*)x, (unsigned char*)xq, xs, total, gpr, ld_x, ld_q,
-                       ld_s);
-  else if (dtype == DLB_DTYPE_F16)
-    hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_F16>, grid, dim3(256), 0, s,
-                       (const unsigned short*)x, (unsigned char*)xq, xs, total, gpr, ld_x, ld_q,
-                       ld_s);
+    hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_BF16>, grid, dim3(kQuantThreads), 0, s, q);
   else
-    return DLB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(quant_fp8_group128_kernel<DLB_DTYPE_F16>, grid, dim3(kQuantThreads), 0, s, q);
   return launch_status();
 }
 
@@ -965,13 +925,21 @@ extern "C" int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, i
   const int64_t total = num_tokens * (N / 8);
   const dim3 grid((uint32_t)ceil_div(total, 256));
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DLB_DTYPE_BF16)
-    hipLaunchKernelGGL(moe_topk_sum_kernel<DLB_DTYPE_BF16>, grid, dim3(256), 0, s,
-                       (const u32x4*)in, (u32x4*)out, total, (int)(N / 8), topk);
-  else if (dtype == DLB_DTYPE_F16)
-    hipLaunchKernelGGL(moe_topk_sum_kernel<DLB_DTYPE_F16>, grid, dim3(256), 0, s,
-                       (const u32x4*)in, (u32x4*)out, total, (int)(N / 8), topk);
-  else
-    return DLB_ERR_UNSUPPORTED;
+  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
+#define DLB_LAUNCH_SUM(DT_, TK_)                                                                  \
+  hipLaunchKernelGGL((moe_topk_sum_kernel<DT_, TK_>), grid, dim3(256), 0, s, (const u32x4*)in, \
+                     (u32x4*)out, total, (int)(N / 8), topk)
+#define DLB_DISPATCH_SUM(DT_)                 \
+  switch (topk) {                             \
+    case 1: DLB_LAUNCH_SUM(DT_, 1); break;    \
+    case 2: DLB_LAUNCH_SUM(DT_, 2); break;    \
+    case 4: DLB_LAUNCH_SUM(DT_, 4); break;    \
+    case 6: DLB_LAUNCH_SUM(DT_, 6); break;    \
+    case 8: DLB_LAUNCH_SUM(DT_, 8); break;    \
+    default: DLB_LAUNCH_SUM(DT_, 0); break;   \
+  }
+  if (dtype == DLB_DTYPE_BF16) { DLB_DISPATCH_SUM(DLB_DTYPE_BF16) } else { DLB_DISPATCH_SUM(DLB_DTYPE_F16) }
+#undef DLB_DISPATCH_SUM
+#undef DLB_LAUNCH_SUM
   return launch_status();
 }

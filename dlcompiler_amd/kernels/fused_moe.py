@@ -15,6 +15,8 @@ from .moe_gating import moe_align_block_size
 # rows per grouped-GEMM workgroup tile = alignment block of the routing; tiles skip 32-row groups
 # that hold padding only, so the matrix work follows the routed rows in steps of 32
 _BLOCK_M = 128
+# block size an alignment handed to fused_moe / fused_moe_fp8 must have been built with
+ALIGN_BLOCK = _BLOCK_M
 
 
 def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
@@ -42,6 +44,58 @@ def per_token_group_quant_fp8(x: torch.Tensor, group_size: int = 128):
                 K // 128, _lib.torch_dtype_code(x.dtype), _lib.current_stream_ptr(x.device))
         _lib.check(st, "dlb_per_token_group_quant_fp8")
     return xq, xs
+
+
+def _align_and_quant(topk_ids: torch.Tensor, block: int, num_experts: int, x: torch.Tensor):
+    """:func:`moe_align_block_size` (with counts) and :func:`per_token_group_quant_fp8` as one
+    native call of two launches: the quantiser runs in the launch of the placement pass.
+    Returns ``(sorted_token_ids, counts, xq, xs)``."""
+    ids = topk_ids.reshape(-1)
+    if ids.dtype != torch.int32:
+        ids = ids.to(torch.int32)
+    ids = ids.contiguous()
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    M, K = x.shape
+    if K % 128 != 0:
+        raise ValueError("K must be a multiple of 128")
+    numel, dev = ids.numel(), ids.device
+    cap = numel + num_experts * (block - 1)
+    nblk = max(1, -(-cap // block))
+    lib = _lib.load()
+    ws_words = max((lib.dlb_moe_align_ws_bytes(numel, num_experts) + 3) // 4, 1)
+    sizes = (cap, nblk, 1, num_experts, ws_words, M * (K // 128))
+    offs, total = [], 0
+    for n in sizes:
+        offs.append(total)
+        total += (n + 3) & ~3
+    buf = torch.empty((total,), dtype=torch.int32, device=dev)
+    sorted_ids, expert_ids, num_post, counts, ws, xs_raw = (buf[o:o + n] for o, n in zip(offs, sizes))
+    xs = xs_raw.view(torch.float32).view(M, K // 128)
+    xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=dev)
+    with _lib.device_guard(dev):
+        st = lib.dlb_moe_align_quant_fp8(
+            ids.data_ptr(), numel, num_experts, block, sorted_ids.data_ptr(), cap,
+            expert_ids.data_ptr(), nblk, counts.data_ptr(), num_post.data_ptr(), ws.data_ptr(),
+            ws.numel() * 4, x.data_ptr(), xq.data_ptr(), xs.data_ptr(), M, K,
+            x.stride(0) if M > 1 else K, K, K // 128, _lib.torch_dtype_code(x.dtype),
+            _lib.current_stream_ptr(dev))
+    _lib.check(st, "dlb_moe_align_quant_fp8")
+    return sorted_ids, counts, xq, xs
+
+
+def _check_alignment(alignment, topk_ids, block, num_experts):
+    """``alignment = (sorted_token_ids, counts)`` as :func:`moe_align_block_size` (or
+    :func:`moe_topk_softmax_align`) returns them for these ``topk_ids`` with ``block_size`` =
+    ``ALIGN_BLOCK`` over all ``num_experts`` experts."""
+    sorted_ids, counts = alignment
+    _lib.require_cuda(sorted_ids, counts)
+    numel = topk_ids.numel()
+    if sorted_ids.dtype != torch.int32 or counts.dtype != torch.int32:
+        raise TypeError("alignment tensors must be int32")
+    if sorted_ids.numel() < numel + num_experts * (block - 1) or counts.numel() != num_experts:
+        raise ValueError(f"alignment does not fit these topk_ids (block {block}, {num_experts} experts)")
+    return sorted_ids.contiguous(), counts.contiguous()
 
 
 def shuffle_moe_weight(w: torch.Tensor) -> torch.Tensor:
@@ -82,7 +136,8 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
                   expert_offset: int = 0,
                   num_experts: int = None,
                   renormalize: bool = False,
-                  weights_shuffled: bool = False) -> torch.Tensor:
+                  weights_shuffled: bool = False,
+                  alignment=None) -> torch.Tensor:
     """fp8 MoE MLP: per-token-group quant -> gate_up grouped GEMM (+SiLU-and-mul, re-quant)
     -> down grouped GEMM (x routing weight) -> sum over the top-k slots.
 
@@ -94,6 +149,11 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     ``expert_offset .. expert_offset + E``; ``num_experts`` the global count (defaults to
     ``E``), as in the reference.  ``weights_shuffled=True`` says ``w1_q``/``w2_q`` went through
     :func:`shuffle_moe_weight_fp8` (same shapes, operand-order bytes) -- the fast path.
+    ``alignment = (sorted_token_ids, counts)`` hands over the expert alignment of ``topk_ids`` a
+    caller already holds (``moe_topk_softmax_align(..., ALIGN_BLOCK, return_counts=True)`` or
+    ``moe_align_block_size(topk_ids, ALIGN_BLOCK, num_experts, return_counts=True)``): the layer
+    then sorts its routing once, in the router, instead of again in here (the reference sorts
+    inside, fused_moe.py:314-320; that is what happens when ``alignment`` is None).
     """
     _lib.require_cuda(hidden_states, w1_q, w1_s, w2_q, w2_s, topk_weights, topk_ids)
     assert hidden_states.dim() == 2 and topk_ids.shape == topk_weights.shape
@@ -119,10 +179,13 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     w2_s = w2_s.to(torch.float32).contiguous()
 
     block = _BLOCK_M
-    sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
-                                                    return_counts=True)
+    if alignment is None:
+        # alignment and activation quantisation: one native call, two launches
+        sorted_ids, counts, xq, xs = _align_and_quant(topk_ids, block, num_experts, hidden_states)
+    else:
+        sorted_ids, counts = _check_alignment(alignment, topk_ids, block, num_experts)
+        xq, xs = per_token_group_quant_fp8(hidden_states)
     num_mblocks = sorted_ids.numel() // block  # whole blocks the slot list can hold
-    xq, xs = per_token_group_quant_fp8(hidden_states)
 
     # one allocation for the intermediates: fp8 rows + their scales (fp32) + the slot outputs
     rows = num_mblocks * block
@@ -163,13 +226,15 @@ def fused_moe(hidden_states: torch.Tensor,
               expert_offset: int = 0,
               num_experts: int = None,
               renormalize: bool = False,
-              weights_shuffled: bool = False) -> torch.Tensor:
+              weights_shuffled: bool = False,
+              alignment=None) -> torch.Tensor:
     """fused moe -- signature and semantics of ``dlblas.kernels.fused_moe.fused_moe``
     (reference: fused_moe.py:296-376): ``w1`` [E, 2I, H] (gate rows first), ``w2`` [E, H, I],
     bf16/f16; routing slots are grouped by expert, the gate_up grouped GEMM runs with the
     SiLU-and-mul fused into its epilogue (same rounding points as the reference), the down
     grouped GEMM applies the routing weight and the top-k slots are summed.
-    ``weights_shuffled`` is this package's extension (see :func:`shuffle_moe_weight`)."""
+    ``weights_shuffled`` and ``alignment`` are this package's extensions (see
+    :func:`shuffle_moe_weight` and :func:`fused_moe_fp8`)."""
     _lib.require_cuda(hidden_states, w1, w2, topk_weights, topk_ids)
     M = hidden_states.size(0)
     E, N, _ = w1.shape
@@ -192,8 +257,11 @@ def fused_moe(hidden_states: torch.Tensor,
     topk_weights = topk_weights.to(torch.float32).contiguous()
 
     block = _BLOCK_M
-    sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
-                                                    return_counts=True)
+    if alignment is None:
+        sorted_ids, _, _, counts = moe_align_block_size(topk_ids, block, num_experts,
+                                                        return_counts=True)
+    else:
+        sorted_ids, counts = _check_alignment(alignment, topk_ids, block, num_experts)
     num_mblocks = sorted_ids.numel() // block  # whole blocks the slot list can hold
     act = torch.empty((num_mblocks * block, I), dtype=dt, device=dev)
     full = (expert_offset == 0 and num_experts == E)

@@ -105,12 +105,13 @@ _FUSED_MAX_TOKENS = 32768  # beyond this the fused entry point declines (DLB_ERR
 
 
 def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_experts: int = None,
-                           renormalize: bool = True):
+                           renormalize: bool = True, return_counts: bool = False):
     """:func:`moe_topk_softmax` followed by :func:`moe_align_block_size` on its ids, as one
     native call of two launches (the router also produces the alignment's per-chunk expert
     counts).  Returns ``(weights, ids, sorted_token_ids, expert_ids, num_tokens_post_padded)``,
-    bit for bit what the two functions return.  More than 32768 tokens, or ``num_experts``
-    different from the router's expert count, take the two separate calls.
+    bit for bit what the two functions return (plus the per-expert ``counts`` with
+    ``return_counts``).  More than 32768 tokens, or ``num_experts`` different from the router's
+    expert count, take the two separate calls.
     """
     assert logits.dim() == 2
     _lib.require_cuda(logits)
@@ -123,7 +124,8 @@ def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_ex
         raise ValueError("block_size must be positive")
     if T > _FUSED_MAX_TOKENS or num_experts != E or k > 16 or E > 256:
         weights, ids = moe_topk_softmax(logits, k, renormalize)
-        return (weights, ids) + tuple(moe_align_block_size(ids, block_size, num_experts))
+        return (weights, ids) + tuple(moe_align_block_size(ids, block_size, num_experts,
+                                                           return_counts=return_counts))
     if logits.dtype != torch.float32:
         logits = logits.float()
     if logits.stride(1) != 1:
@@ -139,21 +141,24 @@ def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_ex
         # one allocation of 4-byte words, carved into the results and the scratch (each piece
         # followed by the padding that keeps the next one 16-byte aligned)
         pieces = []
-        for n in (numel, numel, cap, nblk, 1, ws_words):
+        for n in (numel, numel, cap, nblk, 1, ws_words, E):
             pieces += [n, -n & 3]
         if len(_FUSED_PLANS) > 64:
             _FUSED_PLANS.clear()
         plan = _FUSED_PLANS[(T, E, k, block_size)] = (pieces, sum(pieces))
     pieces, total = plan
     buf = torch.empty((total,), dtype=torch.int32, device=dev)
-    w_raw, _, ids, _, sorted_ids, _, expert_ids, _, num_post, _, ws, _ = buf.split(pieces)
+    w_raw, _, ids, _, sorted_ids, _, expert_ids, _, num_post, _, ws, _, counts, _ = buf.split(pieces)
     weights = w_raw.view(torch.float32).view(T, k)
     ids = ids.view(T, k)
     with _lib.device_guard(dev):
         st = lib.dlb_moe_topk_softmax_align_f32(
             logits.data_ptr(), weights.data_ptr(), ids.data_ptr(), T, E, k,
             logits.stride(0) if T > 1 else E, int(bool(renormalize)), block_size,
-            sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk, None, num_post.data_ptr(),
+            sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk, counts.data_ptr(),
+            num_post.data_ptr(),
             ws.data_ptr(), ws.numel() * 4, _lib.current_stream_ptr(dev))
     _lib.check(st, "dlb_moe_topk_softmax_align_f32")
+    if return_counts:
+        return weights, ids, sorted_ids, expert_ids, num_post, counts
     return weights, ids, sorted_ids, expert_ids, num_post

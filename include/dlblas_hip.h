@@ -103,6 +103,19 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
                              int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
                              void* ws, size_t ws_bytes, void* stream);
 
+/* dlb_moe_align_block_size and dlb_per_token_group_quant_fp8 (declared further down) as one
+ * pipeline of two launches instead of three: the activation quantiser runs in the launch of the
+ * alignment's placement pass (the two jobs are independent).  Arguments and results are those of
+ * the two functions, bit for bit; it is what fused_moe_fp8 runs in front of its GEMMs (the
+ * reference sorts inside fused_moe as well, kernels/fused_moe.py:314-320).  Inputs beyond 524288
+ * routing slots fall back to the separate launches. */
+int dlb_moe_align_quant_fp8(const int32_t* topk_ids, int64_t numel, int E, int block,
+                            int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids,
+                            int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
+                            void* ws, size_t ws_bytes, const void* x, void* xq, float* xs,
+                            int64_t M, int K, int64_t ld_x, int64_t ld_q, int64_t ld_s, int dtype,
+                            void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * dlb_moe_align_block_size without a workspace argument and without any allocation: same
  * arguments, same results bit for bit.  It has no counterpart in the reference; it exists for

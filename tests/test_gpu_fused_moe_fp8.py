@@ -276,3 +276,58 @@ def test_dynamic_range(dev, case):
         out = fm.fused_moe_fp8(*d, k, weights_shuffled=shuffled).cpu()
         assert torch.isfinite(out.float()).all()
         assert _rel_err(out, ref) <= 3e-2, (case, _rel_err(out, ref))
+
+
+# alignment + quantisation as one native call (the quantiser rides in the placement launch) gives
+# what the two separate operators give, bit for bit, across the chunk-size regimes of the alignment
+@pytest.mark.parametrize("T,H,E,k", [(4096, 2048, 64, 6), (1, 128, 8, 2), (77, 384, 60, 6),
+                                     (16384, 256, 64, 6), (300, 1408, 256, 8), (90000, 128, 16, 6)])
+def test_align_and_quant_one_call(dev, T, H, E, k):
+    from dlcompiler_amd.kernels import fused_moe as fm
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size
+
+    g = torch.Generator().manual_seed(T + E)
+    x = (torch.randn((T, H), generator=g) * 3).to(torch.bfloat16).to(dev)
+    ids = torch.randint(0, E, (T, k), generator=g).to(torch.int32).to(dev)
+    sorted_ids, counts, xq, xs = fm._align_and_quant(ids, fm.ALIGN_BLOCK, E, x)
+    rs, _, rn, rc = moe_align_block_size(ids, fm.ALIGN_BLOCK, E, return_counts=True)
+    rq, rsc = fm.per_token_group_quant_fp8(x)
+    assert torch.equal(sorted_ids, rs) and torch.equal(counts, rc)
+    assert torch.equal(xq.view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs, rsc)
+    os_, _, _, oc = og.align_block_size(ids.cpu(), fm.ALIGN_BLOCK, E)
+    npad = int(rn.item())
+    assert torch.equal(sorted_ids.cpu()[:npad], os_[:npad]) and torch.equal(counts.cpu(), oc)
+
+
+# a caller that already holds the alignment of its routing (from the router call) hands it over:
+# same result bit for bit as when fused_moe_fp8 / fused_moe sort the routing themselves
+def test_alignment_handed_over(dev):
+    from dlcompiler_amd.kernels import fused_moe as fm
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size, moe_topk_softmax_align
+
+    T, H, I, E, k = 320, 512, 256, 16, 4
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+    logits = torch.randn((T, E), generator=g)
+    w1 = torch.randn((E, 2 * I, H), generator=g) * 0.05
+    w2 = torch.randn((E, H, I), generator=g) * 0.05
+    w1q, w1s = ofp8.block_quant_weight(w1)
+    w2q, w2s = ofp8.block_quant_weight(w2)
+    tw, ids, sorted_ids, _, _, counts = moe_topk_softmax_align(logits.to(dev), k, fm.ALIGN_BLOCK,
+                                                               return_counts=True)
+    rw, rids = og.topk_softmax(logits, k)
+    assert torch.equal(ids.cpu(), rids)
+    assert torch.equal(counts.cpu(), og.expert_counts(rids, E))
+    d = [t.to(dev) for t in (x, w1q, w1s, w2q, w2s)]
+    base = fm.fused_moe_fp8(*d, tw, ids, k)
+    handed = fm.fused_moe_fp8(*d, tw, ids, k, alignment=(sorted_ids, counts))
+    assert torch.equal(base, handed)
+    _check(base.cpu(), ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, rw, rids))
+    s2, _, _, c2 = moe_align_block_size(ids, fm.ALIGN_BLOCK, E, return_counts=True)
+    b16 = fm.fused_moe(d[0], w1.to(torch.bfloat16).to(dev), w2.to(torch.bfloat16).to(dev), tw, ids, k)
+    h16 = fm.fused_moe(d[0], w1.to(torch.bfloat16).to(dev), w2.to(torch.bfloat16).to(dev), tw, ids, k,
+                       alignment=(s2, c2))
+    assert torch.equal(b16, h16)
+    with pytest.raises(ValueError):      # an alignment built with another block size does not fit
+        s64, _, _, c64 = moe_align_block_size(ids, 8, E, return_counts=True)
+        fm.fused_moe_fp8(*d, tw, ids, k, alignment=(s64, c64))
