@@ -56,6 +56,9 @@ SIGNATURES = {
     "dlb_moe_gemm_16bit_gate_up": (c_int, [c_void_p] * 4 + [c_int] * 10 + [c_void_p, c_int, c_void_p]),
     "dlb_moe_gemm_16bit_down": (c_int, [c_void_p] * 4 + [c_int, c_void_p] + [c_int] * 9
                                 + [c_void_p, c_int, c_void_p]),
+    "dlb_moe_gemm_16bit_launcher": (c_int, [c_void_p] * 6 + [c_int, c_void_p, c_int, c_int, c_int,
+                                                            c_int64, c_int64] + [c_int] * 6
+                                    + [c_void_p]),
     "dlb_fill_kv_cache": (c_int, [c_void_p] * 8 + [c_int, c_int64] + [c_int] * 7 + [c_int64] * 11
                           + [c_void_p]),
     "dlb_rms_norm": (c_int, [c_void_p] * 5 + [c_int64, c_int] + [c_int64] * 4

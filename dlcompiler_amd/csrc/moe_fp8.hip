@@ -60,8 +60,14 @@ struct MoeGemmParams {
   const float* a_scale;       // [rows, K / 128]
   const unsigned char* w;     // weights [E_local, N, K]
   const float* w_scale;       // [E_local, N / 128, K / 128]
-  const int32_t* sorted_ids;  // [num_mblocks * block_m] routing slots grouped by expert
-  const int32_t* counts;      // [num_experts] routed slots per (global) expert
+  IdxArray sorted_ids;        // [num_mblocks * block_m] routing slots grouped by expert
+  IdxArray counts;            // [num_experts] routed slots per (global) expert
+  // launcher form of the routing (non-gated kernel only): the slot list is NOT padded per expert;
+  // expert e owns its positions seg_start[e] .. counts[e] - 1 (counts then holds the segment ENDS)
+  IdxArray seg_start;         // p == nullptr: block-aligned list
+  int64_t a_rows;             // rows of `a` when it is read in sorted order (reads are clamped to it)
+  int gather_a;               // non-gated kernel: rows of `a` are gathered by token (slot / topk)
+  int scatter_c;              // non-gated kernel: output row = routing slot (else the sorted position)
   int num_experts;            // global expert count = length of counts
   int num_mblocks;            // capacity of sorted_ids in blocks
   int bm_shift;               // log2(block_m): 6 or 7
@@ -130,18 +136,20 @@ __device__ __forceinline__ void wait_vm() {
 // and two wave scans.  All results are wave-uniform.
 struct TileId {
   int e;     // local expert
-  int mb;    // block index into sorted_ids
+  int row0;  // first position of the tile's rows in sorted_ids
   int nt;    // column tile
   int rows;  // real (unpadded) rows of the block, 1 .. block_m
 };
 __device__ __forceinline__ bool find_tile(const MoeGemmParams& p, int lane, TileId& t) {
   const int bm = 1 << p.bm_shift;
-  int cnt[4], nb[4], tl[4];
+  const bool segs = p.seg_start.p != nullptr;
+  int cnt[4], nb[4], tl[4], st[4];
   int nb_sum = 0, tl_sum = 0;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int e = 4 * lane + c;
-    cnt[c] = e < p.num_experts ? max(p.counts[e], 0) : 0;
+    st[c] = (segs && e < p.num_experts) ? p.seg_start[e] : 0;
+    cnt[c] = e < p.num_experts ? max(p.counts[e] - st[c], 0) : 0;
     nb[c] = (cnt[c] + bm - 1) >> p.bm_shift;
     const bool local = e >= p.expert_offset && e < p.expert_offset + p.num_local;
     tl[c] = local ? nb[c] * p.num_ntiles : 0;
@@ -159,19 +167,21 @@ __device__ __forceinline__ bool find_tile(const MoeGemmParams& p, int lane, Tile
   const int L = __builtin_ctzll(hit);  // the lane whose four experts hold the tile
   int rem = logical - __builtin_amdgcn_readlane(tl_incl - tl_sum, L);
   int mbase = __builtin_amdgcn_readlane(nb_incl - nb_sum, L);
-  int e = 4 * L, nbe = 1, ce = 0;
+  int e = 4 * L, nbe = 1, ce = 0, se = 0;
   bool found = false;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int tc = __builtin_amdgcn_readlane(tl[c], L);
     const int nc = __builtin_amdgcn_readlane(nb[c], L);
     const int cc = __builtin_amdgcn_readlane(cnt[c], L);
+    const int sc = __builtin_amdgcn_readlane(st[c], L);
     if (!found) {
       if (rem < tc) {
         found = true;
         e = 4 * L + c;
         nbe = nc;
         ce = cc;
+        se = sc;
       } else {
         rem -= tc;
         mbase += nc;
@@ -181,10 +191,12 @@ __device__ __forceinline__ bool find_tile(const MoeGemmParams& p, int lane, Tile
   const int nt = rem / nbe;
   const int rb = rem - nt * nbe;
   t.e = e - p.expert_offset;
-  t.mb = mbase + rb;
+  // block-aligned list: block mbase + rb; launcher form: the expert's own segment
+  t.row0 = segs ? se + (rb << p.bm_shift) : (mbase + rb) << p.bm_shift;
   t.nt = nt;
   t.rows = min(bm, ce - (rb << p.bm_shift));
-  return t.mb < p.num_mblocks;  // (counts that do not fit the slot list: touch nothing)
+  // (counts that do not fit the slot list: touch nothing)
+  return segs ? t.row0 + t.rows <= p.numel : (mbase + rb) < p.num_mblocks;
 }
 
 // QT = 0: fp8 operands with block scales; QT = 1: 16-bit operands of type DT, no scales.
@@ -261,7 +273,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
   constexpr int NRT = decltype(nrt_tag)::value;
   const int e = tile.e, nt = tile.nt;
   const int nrt_real = (tile.rows + 31) >> 5;  // row tiles that hold real rows (<= NRT)
-  const int row0 = tile.mb << p.bm_shift;
+  const int row0 = tile.row0;
   const int K = p.K, KC = p.KC;
   const bool stager = wave < nrt_real;  // this wave's row tile is real: it stages those rows
 
@@ -306,29 +318,36 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
   // fetches.  Down: thread t < 128 keeps slot and routing weight of row t for the epilogue.
   int sid_x[4] = {0, 0, 0, 0};
   int sid_s = 0;
-  if (GATED) {
-    if (stager) {
+  // (positions past the tile's real rows hold the pad sentinel in a block-aligned list and another
+  // expert's slots in the launcher form: they are not read)
+  auto slot_at = [&](int r) -> int { return r < tile.rows ? p.sorted_ids[row0 + r] : p.numel; };
+  const bool gather = GATED || p.gather_a;
+  if (gather && stager) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sid_x[i] = p.sorted_ids[row0 + 32 * wave + 8 * i + drow];
-      if (QT == 0) sid_s = p.sorted_ids[row0 + 32 * wave + j];
-    }
-  } else {
+    for (int i = 0; i < 4; ++i) sid_x[i] = slot_at(32 * wave + 8 * i + drow);
+    if (QT == 0) sid_s = slot_at(32 * wave + j);
+  }
+  if (!GATED) {
     if (tid < 128) {
-      int sid = p.numel;
+      // destination row of the tile's row `tid` (-1: none) and its routing weight
+      int dst = -1;
       float rwt = 0.0f;
-      if (tid < 32 * nrt_real) {
-        sid = p.sorted_ids[row0 + tid];
-        if (sid < p.numel) rwt = p.topk_w[sid];
+      if (tid < tile.rows) {
+        const int sid = p.sorted_ids[row0 + tid];
+        if (sid >= 0 && sid < p.numel) {
+          dst = p.scatter_c ? sid : row0 + tid;
+          rwt = p.topk_w ? p.topk_w[sid] : 1.0f;
+        }
       }
-      sid_lds[tid] = sid;  // published by the barrier that opens the main loop
+      sid_lds[tid] = dst;  // published by the barrier that opens the main loop
       rw_lds[tid] = rwt;
     }
   }
   // source row of the tile's row r whose routing slot is sid (gated: the slot's token; pad
   // slots read a valid row)
   auto src_row_of = [&](int sid, int r) -> uint32_t {
-    if (GATED) return (uint32_t)min(sid / p.topk, p.num_tokens - 1);
-    return (uint32_t)(row0 + r);
+    if (gather) return (uint32_t)min(max(sid, 0) / p.topk, p.num_tokens - 1);
+    return (uint32_t)min((int64_t)(row0 + r), p.a_rows - 1);
   };
   // ---- activation staging: per chunk 16 instructions of 8 rows x 128 bytes, four per wave
   // (its own row tile); lane -> (row, physical piece), the logical piece it fetches undoes the
@@ -677,8 +696,8 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const int r = (tid_e >> 5) + 8 * i, pc = tid_e & 31;
-          const int sid = sid_lds[64 * half + r];
-          if (sid < p.numel && 8 * pc < ncols)
+          const int sid = sid_lds[64 * half + r];  // destination row
+          if (sid >= 0 && 8 * pc < ncols)
             // (non-temporal: the 100 MB of slot rows would otherwise push the weight lines that the
             // expert's other row blocks are about to read out of L2)
             __builtin_nontemporal_store(
@@ -818,8 +837,12 @@ int fill_gemm_params(MoeGemmParams& p, bool gated, int elem, const void* a, cons
   p.a_scale = a_scale;
   p.w = (const unsigned char*)w;
   p.w_scale = w_scale;
-  p.sorted_ids = sorted_ids;
-  p.counts = expert_counts;
+  p.sorted_ids = IdxArray{sorted_ids, 0};
+  p.counts = IdxArray{expert_counts, 0};
+  p.seg_start = IdxArray{nullptr, 0};
+  p.a_rows = a_rows;
+  p.gather_a = 0;   // (the gated kernel always gathers; the down GEMMs read sorted rows)
+  p.scatter_c = 1;
   p.num_experts = num_experts;
   p.num_mblocks = num_mblocks;
   p.bm_shift = block_m == 128 ? 7 : 6;
@@ -913,6 +936,61 @@ extern "C" int dlb_moe_gemm_16bit_down(const void* act, const void* w2,
   p.out = out;
   p.topk_w = topk_weights;
   return launch_moe_gemm<false, 1>(p, dtype, w_layout, (hipStream_t)stream);
+}
+
+// The reference's grouped-GEMM launcher in its own argument form (16-bit operands):
+// C[row] = A[row'] . B[e]^T (x weights[slot]) for every routing slot of the expert-sorted list.
+extern "C" int dlb_moe_gemm_16bit_launcher(const void* a, const void* b, void* c,
+                                           const void* sorted_idx, const void* exp_start,
+                                           const void* exp_end, int index64_mask,
+                                           const float* weights, int num_experts,
+                                           int expert_offset, int num_local_experts,
+                                           int64_t num_slots, int64_t a_rows, int topk, int N,
+                                           int K, int reindex_a, int reindex_c, int dtype,
+                                           void* stream) {
+  using namespace dlb;
+  if (num_slots < 0 || a_rows < 0 || topk < 1 || N < 1 || K < 1) return DLB_ERR_BAD_ARG;
+  if (num_experts < 1 || num_local_experts < 1 || expert_offset < 0 ||
+      expert_offset + num_local_experts > num_experts)
+    return DLB_ERR_BAD_ARG;
+  if (index64_mask & ~7) return DLB_ERR_BAD_ARG;
+  if (num_slots == 0) return DLB_OK;
+  if (!a || !b || !c || !sorted_idx || !exp_start || !exp_end || a_rows < 1) return DLB_ERR_BAD_ARG;
+  if (num_experts > 256) return DLB_ERR_UNSUPPORTED;
+  if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
+  // rows are whole 128-byte chunks (64 elements); outputs leave in 16-byte pieces
+  if (K % 64 != 0 || N % 8 != 0) return DLB_ERR_UNSUPPORTED;
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return DLB_ERR_UNSUPPORTED;
+  if ((int64_t)N * K * 2 >= (int64_t)0xffffffffu || a_rows * K * 2 >= (int64_t)0xffffffffu ||
+      num_slots >= (int64_t)0x7fffffff)
+    return DLB_ERR_UNSUPPORTED;
+  MoeGemmParams p = MoeGemmParams{};
+  p.a = (const unsigned char*)a;
+  p.w = (const unsigned char*)b;
+  p.sorted_ids = idx_array(sorted_idx, index64_mask, 0);
+  p.seg_start = idx_array(exp_start, index64_mask, 1);
+  p.counts = idx_array(exp_end, index64_mask, 2);   // segment ends: find_tile subtracts the starts
+  p.num_experts = num_experts;
+  p.bm_shift = 7;
+  // every expert's segment is cut into blocks of 128 rows of its own: at most one partial block each
+  p.num_mblocks = (int)(ceil_div(num_slots, 128) + num_local_experts);
+  p.num_ntiles = (int)ceil_div(N, 256);
+  p.K = K * 2;
+  p.N = N;
+  p.KC = p.K / 128;
+  p.topk = topk;
+  p.numel = (int)num_slots;
+  // gathered rows are slot / topk; the caller says how many rows `a` has
+  p.num_tokens = a_rows < 0x7fffffff ? (int)a_rows : 0x7fffffff;
+  p.a_rows = a_rows;
+  p.expert_offset = expert_offset;
+  p.num_local = num_local_experts;
+  p.I = 0;
+  p.gather_a = reindex_a ? 1 : 0;
+  p.scatter_c = reindex_c ? 1 : 0;
+  p.out = c;
+  p.topk_w = weights;  // null: no routing weights
+  return launch_moe_gemm<false, 1>(p, dtype, 0, (hipStream_t)stream);
 }
 
 extern "C" int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk,

@@ -125,6 +125,50 @@ def get_start_end(topk_idx: torch.Tensor, sorted_idx: torch.Tensor, num_experts:
     return exp_start, exp_end
 
 
+def fused_moe_kernel_launcher(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    C: torch.Tensor,
+    sorted_idx: torch.Tensor,
+    exp_start: torch.Tensor,
+    exp_end: torch.Tensor,
+    weights: torch.Tensor,
+    enable_weights: bool = False,
+    top_k: int = 1,
+    num_tokens: int = None,
+    expert_offset: int = 0,
+    reindex_a: bool = True,
+    reindex_c: bool = True,
+):
+    """fused moe kernel launcher -- signature and semantics of
+    ``dlblas.kernels.fused_moe.fused_moe_kernel_launcher`` (reference: fused_moe.py:178-235): the
+    grouped GEMM ``C[row] = A[row'] @ B[e].T`` over the expert-sorted slot list
+    (``sorted_idx = topk_ids.flatten().argsort()``, ``exp_start``/``exp_end`` from
+    :func:`get_start_end`), rows gathered by token (``reindex_a``), scattered to their slot
+    (``reindex_c``) and scaled by ``weights`` (``enable_weights``).  Writes ``C`` in place.
+    ``num_tokens`` only sizes the reference's grid and is ignored here."""
+    _lib.require_cuda(A, B, C, sorted_idx, exp_start, exp_end)
+    A2, C2 = A.flatten(0, -2), C.flatten(0, -2)
+    E, N, K = B.shape
+    assert A2.shape[1] == K and C2.shape[1] == N and A.dtype == B.dtype == C.dtype
+    assert A2.is_contiguous() and C2.is_contiguous() and B.is_contiguous()
+    assert C2.data_ptr() == C.data_ptr()
+    w = None
+    if enable_weights:
+        w = weights.reshape(-1).to(torch.float32).contiguous()
+    (sorted_idx, exp_start, exp_end), mask = _lib.index_arrays(
+        sorted_idx.contiguous(), exp_start.contiguous(), exp_end.contiguous())
+    lib = _lib.load()
+    with _lib.device_guard(A.device):
+        st = lib.dlb_moe_gemm_16bit_launcher(
+            A2.data_ptr(), B.data_ptr(), C2.data_ptr(), sorted_idx.data_ptr(), exp_start.data_ptr(),
+            exp_end.data_ptr(), mask, w.data_ptr() if w is not None else None, exp_start.numel(),
+            int(expert_offset), E, sorted_idx.numel(), A2.shape[0], int(top_k), N, K,
+            int(bool(reindex_a)), int(bool(reindex_c)), _lib.torch_dtype_code(A.dtype),
+            _lib.current_stream_ptr(A.device))
+    _lib.check(st, "dlb_moe_gemm_16bit_launcher")
+
+
 def fused_moe_fp8(hidden_states: torch.Tensor,
                   w1_q: torch.Tensor,
                   w1_s: torch.Tensor,

@@ -334,6 +334,25 @@ int dlb_moe_gemm_16bit_down(const void* act, const void* w2, const int32_t* sort
                             int num_local_experts, int w_layout, void* out, int dtype,
                             void* stream);
 
+/* The reference's grouped-GEMM launcher in its own argument form: replaces fused_moe_kernel +
+ * fused_moe_kernel_launcher, kernels/fused_moe.py:82-235 (16-bit operands, fp32 accumulation).
+ *   a [a_rows, K], b [num_local_experts, N, K] (row-major), c [rows, N], all of `dtype`
+ *   sorted_idx [num_slots]: the flat routing slots (token * topk + j) sorted by expert, NOT padded
+ *   exp_start / exp_end [num_experts]: expert e owns sorted positions exp_start[e] .. exp_end[e] - 1
+ *     (:267-293); local expert i is global expert expert_offset + i (:113-114)
+ *   the three index arrays are int32 or int64 (index64_mask bit 0 = sorted_idx, 1 = exp_start,
+ *   2 = exp_end; the reference passes the int64 result of argsort)
+ *   for sorted position p with slot s = sorted_idx[p] of expert e:
+ *     c[reindex_c ? s : p, :] = (a[reindex_a ? s / topk : p, :] . b[e]^T) * (weights ? weights[s] : 1)
+ *   rounded once to `dtype` (:119-175); rows of c that no slot maps to are not written.
+ * K % 64 == 0 (whole 128-byte chunks), N % 8 == 0, 16-byte aligned pointers, num_experts <= 256. */
+int dlb_moe_gemm_16bit_launcher(const void* a, const void* b, void* c, const void* sorted_idx,
+                                const void* exp_start, const void* exp_end, int index64_mask,
+                                const float* weights, int num_experts, int expert_offset,
+                                int num_local_experts, int64_t num_slots, int64_t a_rows, int topk,
+                                int N, int K, int reindex_a, int reindex_c, int dtype,
+                                void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Decoder-layer helpers around the attention / MoE kernels (memory-bound).
  * ---------------------------------------------------------------------------------------- */

@@ -48,6 +48,26 @@ def fused_moe(hidden, w1, w2, topk_weights, topk_ids, renormalize=False, expert_
     return slots.float().sum(dim=1).to(dt)                       # :375
 
 
+def grouped_gemm_launcher(A, B, topk_idx, weights=None, expert_offset=0):
+    """Ground truth of the reference's launcher test,
+    python/dlBLAS/tests/kernels/test_fused_moe.py:97-112: ``C[t, j] = A[t] @ B[e].T`` for the
+    expert ``e = topk_idx[t, j]`` (optionally times ``weights[t, j]``), returned flattened to
+    ``[tokens * top_k, N]`` in slot order; slots of experts outside
+    ``[expert_offset, expert_offset + B.shape[0])`` stay zero.  Products accumulate in fp32 and
+    are rounded once to the operand type (kernel: fused_moe.py:148-166)."""
+    M, top_k = topk_idx.shape
+    E, N, _ = B.shape
+    C = torch.zeros((M, top_k, N), dtype=torch.float32)
+    for e in range(E):
+        tok, j = torch.where(topk_idx == e + expert_offset)
+        if tok.numel() == 0:
+            continue
+        C[tok, j] = A[tok].float() @ B[e].float().t()
+    if weights is not None:
+        C = C * weights.float()[..., None]
+    return C.to(A.dtype).flatten(0, 1)
+
+
 def fused_moe_fp8(hidden, w1_q, w1_s, w2_q, w2_s, topk_weights, topk_ids, renormalize=False,
                   expert_offset=0):
     """fp8 MoE MLP as a dequantised fp32 evaluation; returns [T, H] in hidden.dtype."""

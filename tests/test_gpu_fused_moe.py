@@ -107,3 +107,61 @@ def test_output_width_comes_from_w2(dev, out_size):
     assert out.shape == (T, out_size)
     scale = max(1.0, ref.float().abs().max().item())
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2 * scale)
+
+
+def _launcher_case(dev, M, K, N, E, top_k, dtype, seed=0, enable_weights=True, reindex_a=True,
+                   reindex_c=True, idx_dtype=torch.int64, local=None):
+    from dlcompiler_amd.kernels.fused_moe import fused_moe_kernel_launcher, get_start_end
+
+    g = torch.Generator().manual_seed(seed)
+    A = ((torch.rand((M, K), generator=g) - 0.5) / 2).to(dtype)        # test_fused_moe.py:49-57
+    B = ((torch.rand((E, N, K), generator=g) - 0.5) / 2).to(dtype)
+    router = torch.rand((M, E), generator=g).to(dtype)
+    weights, topk_idx = router.topk(top_k, dim=-1)
+    sorted_idx = topk_idx.flatten().argsort(stable=True)                # :9-14
+    off, nloc = local if local else (0, E)
+    ref = ofm.grouped_gemm_launcher(A, B[off:off + nloc], topk_idx, weights if enable_weights else None,
+                                    expert_offset=off)
+    ids_d = topk_idx.to(dev)
+    exp_start, exp_end = get_start_end(ids_d, sorted_idx.to(idx_dtype).to(dev), E)
+    Ad = A.to(dev)
+    if not reindex_a:                     # A already holds one row per sorted position
+        Ad = A[sorted_idx // top_k].to(dev)
+    C = torch.full((M * top_k, N), 7.0, dtype=dtype, device=dev)
+    fused_moe_kernel_launcher(Ad, B[off:off + nloc].to(dev), C, sorted_idx.to(idx_dtype).to(dev),
+                              exp_start, exp_end, weights.to(dev), enable_weights=enable_weights,
+                              top_k=top_k, num_tokens=M, expert_offset=off, reindex_a=reindex_a,
+                              reindex_c=reindex_c)
+    out = C.cpu()
+    if not reindex_c:                     # rows in sorted order -> back to slot order
+        back = torch.empty_like(out)
+        back[sorted_idx] = out
+        out = back
+    owned = ((topk_idx >= off) & (topk_idx < off + nloc)).flatten()
+    torch.testing.assert_close(out[owned], ref[owned])               # the reference's own tolerance
+    assert (out[~owned] == 7.0).all()                                # other experts' rows untouched
+
+
+def test_reference_launcher_case(dev):
+    # test_fused_moe.py:17-145: M 256, K 64, N 128, 4 experts, top-2, fp16, weights enabled
+    _launcher_case(dev, 256, 64, 128, 4, 2, torch.float16)
+
+
+@pytest.mark.parametrize("reindex_a,reindex_c", [(True, False), (False, True), (False, False)])
+def test_launcher_reindex_flags(dev, reindex_a, reindex_c):
+    # the two calls of fused_moe: gather + sorted rows (fused_moe.py:334-349), sorted + scatter (:358-373)
+    _launcher_case(dev, 300, 128, 136, 8, 2, torch.bfloat16, seed=1, reindex_a=reindex_a,
+                   reindex_c=reindex_c, enable_weights=reindex_c)
+
+
+@pytest.mark.parametrize("M,K,N,E,k,dtype,idx", [(1, 64, 8, 2, 1, torch.float16, torch.int32),
+                                                 (777, 192, 200, 64, 6, torch.bfloat16, torch.int64),
+                                                 (2000, 256, 512, 16, 4, torch.float16, torch.int32),
+                                                 (130, 2048, 264, 3, 2, torch.bfloat16, torch.int64)])
+def test_launcher_shapes(dev, M, K, N, E, k, dtype, idx):
+    _launcher_case(dev, M, K, N, E, k, dtype, seed=M, idx_dtype=idx)
+    _launcher_case(dev, M, K, N, E, k, dtype, seed=M + 1, idx_dtype=idx, enable_weights=False)
+
+
+def test_launcher_expert_shard(dev):
+    _launcher_case(dev, 400, 128, 128, 8, 2, torch.float16, seed=3, local=(2, 4))

@@ -121,3 +121,24 @@ def test_expert_offset_selects_a_shard():
     lo = ofm.fused_moe(x, w1b[:2], w2b[:2], tw, ids, expert_offset=0).float()
     hi = ofm.fused_moe(x, w1b[2:], w2b[2:], tw, ids, expert_offset=2).float()
     torch.testing.assert_close(lo + hi, full, rtol=2e-2, atol=2e-2)
+
+
+def test_grouped_gemm_launcher_is_a_dense_one_hot_product():
+    # pins oracle.fused_moe.grouped_gemm_launcher (test_fused_moe.py:97-112) with an fp64 dense
+    # evaluation: C[t, j] = sum_e onehot[t, j, e] * (A[t] @ B[e].T) * w[t, j]
+    from oracle import fused_moe as ofm
+
+    g = torch.Generator().manual_seed(4)
+    M, K, N, E, k = 40, 64, 24, 5, 2
+    A = torch.randn((M, K), generator=g)
+    B = torch.randn((E, N, K), generator=g)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(M)])
+    w = torch.rand((M, k), generator=g)
+    got = ofm.grouped_gemm_launcher(A, B, idx, w)
+    dense = torch.einsum("mk,enk->men", A.double(), B.double())               # [M, E, N]
+    ref = torch.gather(dense, 1, idx[..., None].expand(M, k, N)) * w.double()[..., None]
+    torch.testing.assert_close(got.double(), ref.flatten(0, 1), rtol=1e-5, atol=1e-5)
+    part = ofm.grouped_gemm_launcher(A, B[2:4], idx, None, expert_offset=2)   # a shard of experts
+    mask = ((idx >= 2) & (idx < 4)).flatten()
+    full = ofm.grouped_gemm_launcher(A, B, idx, None)
+    assert torch.equal(part[mask], full[mask]) and (part[~mask] == 0).all()
