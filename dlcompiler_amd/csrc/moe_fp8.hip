@@ -544,6 +544,10 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
     x_tgt = xr;
   };
   // two chunks per iteration, so that every weight unit has a fixed home in the register file
+  // The wave runs its main loop at a raised priority: when the CU's other workgroup is in its
+  // prologue or epilogue (vector arithmetic, no matrix work), this wave's MFMAs win the issue slot
+  // they share (gate_up 2 - 3 % faster, down unchanged).
+  __builtin_amdgcn_s_setprio(3);
   int k = 0;
 #pragma nounroll
   for (; k + 1 < KC; k += 2) {
@@ -551,6 +555,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
     chunk(std::integral_constant<int, 1>{}, k + 1);
   }
   if (k < KC) chunk(std::integral_constant<int, 0>{}, k);
+  __builtin_amdgcn_s_setprio(0);
   // the clamped copies past the end are still in flight and will write the LDS slots
   wait_vm<0>();
   // the accumulators hold sum / s(last chunk), whose scales are still in their LDS slot (x_tgt
