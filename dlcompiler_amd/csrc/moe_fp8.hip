@@ -610,7 +610,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const MoeGemmParams p)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {  // 128 rows x 16 pieces of 16 bytes
       const int r = (tid_e >> 4) + 16 * i, pc = tid_e & 15;
-      if (r < 32 * NRT)
+      if (r < 32 * NRT && nt * 128 + 8 * pc < p.I)  // (the last column tile may be partial)
         *(u32x4*)((unsigned short*)p.hq + (int64_t)(row0 + r) * p.I + nt * 128 + 8 * pc) =
             *(const u32x4*)(x_lds + r * kActPitch + 16 * pc);
     }
@@ -793,6 +793,7 @@ template <bool GATED, int QT>
 int launch_moe_gemm(const MoeGemmParams& p, int dtype, int w_layout, hipStream_t s) {
   // one workgroup per tile slot of the block capacity; a workgroup finds its tile from the
   // expert counts (or finds none and leaves), in the order described at find_tile
+  if (w_layout && p.N % 16 != 0) return DLB_ERR_UNSUPPORTED;  // operand order comes in 16-row tiles
   const uint32_t grid = (uint32_t)(ceil_div((int64_t)p.num_mblocks * p.num_ntiles, 8) * 8);
 #define DLB_LAUNCH_GEMM(DT_)                                                                   \
   do {                                                                                       \
@@ -826,8 +827,11 @@ int fill_gemm_params(MoeGemmParams& p, bool gated, int elem, const void* a, cons
   if (expert_offset < 0 || expert_offset + num_local_experts > num_experts) return DLB_ERR_BAD_ARG;
   if (num_experts > 256) return DLB_ERR_UNSUPPORTED;  // four experts per lane in the tile look-up
   if (block_m != 64 && block_m != 128) return DLB_ERR_UNSUPPORTED;
-  // a row must be a whole number of 128-byte chunks; output tiles are 128 columns wide
-  if ((Kel * elem) % 128 != 0 || I % 128 != 0 || H % 128 != 0) return DLB_ERR_UNSUPPORTED;
+  // a row must be a whole number of 128-byte chunks.  fp8: the scale groups and the re-quantised
+  // column tiles are 128 wide; 16 bit: a partial last column tile is masked, so 64-element
+  // multiples do (both reduction lengths) and the output width only has to fill 16-byte stores
+  if (elem == 1 ? (H % 128 != 0 || I % 128 != 0) : (Kel % 64 != 0 || I % 64 != 0 || H % 8 != 0))
+    return DLB_ERR_UNSUPPORTED;
   // fp8: the block scales of all K chunks of a tile are parked in LDS
   if (elem == 1 && Kel / 128 > kMoeMaxKChunks) return DLB_ERR_UNSUPPORTED;
   if (!aligned16(a) || !aligned16(w)) return DLB_ERR_UNSUPPORTED;
@@ -851,7 +855,7 @@ int fill_gemm_params(MoeGemmParams& p, bool gated, int elem, const void* a, cons
   p.num_experts = num_experts;
   p.num_mblocks = num_mblocks;
   p.bm_shift = block_m == 128 ? 7 : 6;
-  p.num_ntiles = gated ? I / 128 : (int)ceil_div(H, 256);
+  p.num_ntiles = gated ? (int)ceil_div(I, 128) : (int)ceil_div(H, 256);
   p.K = Kel * elem;
   p.N = N;
   p.KC = p.K / 128;

@@ -319,7 +319,9 @@ int dlb_moe_topk_sum(const void* in, void* out, int64_t num_tokens, int topk, in
  *            sorted position r -- the rounding points of the reference (GEMM result stored in
  *            the activation dtype, then F.silu(...) * up, :351-352); act [num_mblocks*block_m, I]
  *   down:    out[slot, :] = round((act_r W_down^T) * topk_weights[slot]), out [T * topk, H]
- * x [T, H], w1 [E_local, 2I, H], w2 [E_local, H, I], all of `dtype`; H % 128 == 0, I % 128 == 0.
+ * x [T, H], w1 [E_local, 2I, H], w2 [E_local, H, I], all of `dtype`; the hidden size of the
+ * gate_up call and I multiples of 64 (whole 128-byte chunks; the reference masks any size,
+ * kernels/fused_moe.py:119-160), the output width of the down call a multiple of 8.
  * Follow with dlb_moe_topk_sum.
  * ---------------------------------------------------------------------------------------- */
 int dlb_moe_gemm_16bit_gate_up(const void* x, const void* w1, const int32_t* sorted_ids,

@@ -81,3 +81,26 @@ def test_moe_gemm_argument_checks_need_no_gpu():
     assert lib.dlb_moe_gemm_fp8_gate_up(one, one, one, one, one, None, 8, 4, 128, 64, 2, 256, 128,
                                         0, 8, 1, one, one, None) == -1   # counts are required
     assert lib.dlb_moe_align_block_size_static_max_numel() == 256 * 2048
+
+
+def test_launcher_and_fused_prepare_argument_checks_need_no_gpu():
+    lib = _lib.load()
+    one = 16
+
+    def launcher(K=64, N=128, num_experts=4, offset=0, local=4, slots=512, mask=0):
+        return lib.dlb_moe_gemm_16bit_launcher(one, one, one, one, one, one, mask, None, num_experts,
+                                               offset, local, slots, 256, 2, N, K, 1, 1, 1, None)
+
+    assert launcher(slots=0) == 0                 # nothing to do
+    assert launcher(K=48) == -2                   # rows are whole 128-byte chunks
+    assert launcher(N=12) == -2                   # outputs leave in 16-byte pieces
+    assert launcher(offset=2, local=4) == -1      # local experts outside the global range
+    assert launcher(mask=8) == -1                 # three index arrays: bits 0..2
+    assert launcher(num_experts=300, local=300) == -2
+    # alignment + quantisation in one call: the checks of both halves apply before any launch
+    assert lib.dlb_moe_align_quant_fp8(one, 64, 8, 128, one, 64 + 8 * 127, one, 9, one, one, None, 0,
+                                       one, one, one, 32, 256, 256, 256, 2, 0, None) == -4  # no workspace
+    assert lib.dlb_moe_align_quant_fp8(one, 64, 8, 128, one, 10, one, 9, one, one, one, 1 << 20,
+                                       one, one, one, 32, 256, 256, 256, 2, 0, None) == -1  # sorted_cap too small
+    assert lib.dlb_moe_align_quant_fp8(one, 64, 8, 128, one, 64 + 8 * 127, one, 9, one, one, one, 1 << 20,
+                                       one, one, one, 32, 200, 200, 200, 1, 0, None) == -2  # K % 128

@@ -165,3 +165,28 @@ def test_launcher_shapes(dev, M, K, N, E, k, dtype, idx):
 
 def test_launcher_expert_shard(dev):
     _launcher_case(dev, 400, 128, 128, 8, 2, torch.float16, seed=3, local=(2, 4))
+
+
+# sizes that are multiples of 64 but not of 128 (the last gate / up column tile and the last
+# output tile are partial), output width a multiple of 8; the reference masks any size
+# (fused_moe.py:119-160)
+@pytest.mark.parametrize("T,H,I,O,E,k", [(100, 192, 320, 192, 4, 2), (257, 64, 64, 8, 8, 2),
+                                         (300, 448, 192, 136, 16, 4)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_sizes_that_are_not_multiples_of_128(dev, T, H, I, O, E, k, dtype):
+    from dlcompiler_amd.kernels import fused_moe as fm
+
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn((T, H), generator=g).to(dtype)
+    w1 = (torch.randn((E, 2 * I, H), generator=g) * 0.05).to(dtype)
+    w2 = (torch.randn((E, O, I), generator=g) * 0.05).to(dtype)
+    tw, ids = og.topk_softmax(torch.randn((T, E), generator=g), k)
+    ref = ofm.fused_moe(x, w1, w2, tw, ids)
+    out = fm.fused_moe(x.to(dev), w1.to(dev), w2.to(dev), tw.to(dev), ids.to(dev), k).cpu()
+    assert out.shape == (T, O)
+    scale = max(1.0, ref.float().abs().max().item())
+    torch.testing.assert_close(out.float(), ref.float(), rtol=2e-2, atol=2e-2 * scale)
+    if O % 16 == 0:   # operand-order weights come in 16-row tiles
+        sh = fm.fused_moe(x.to(dev), fm.shuffle_moe_weight(w1.to(dev)), fm.shuffle_moe_weight(w2.to(dev)),
+                          tw.to(dev), ids.to(dev), k, weights_shuffled=True).cpu()
+        assert torch.equal(sh, out)
