@@ -114,6 +114,33 @@ def shuffle_moe_weight(w: torch.Tensor) -> torch.Tensor:
 
 shuffle_moe_weight_fp8 = shuffle_moe_weight
 
+# Operand-order copies made on behalf of callers that hand over the reference's row-major weights
+# on every call and cannot re-arrange them at load time themselves (a patched serving engine):
+# keyed by the weight tensor's storage, dropped when the tensor is modified in place.
+_OPERAND_ORDER_CACHE = {}
+_CACHE_ENV = "DLBLAS_HIP_CACHE_OPERAND_ORDER"
+
+
+def _cache_requested(flag) -> bool:
+    import os
+
+    return bool(flag) if flag is not None else os.environ.get(_CACHE_ENV, "0") not in ("", "0")
+
+
+def _operand_order_cached(w: torch.Tensor) -> torch.Tensor:
+    """The operand-order copy of ``w`` (see :func:`shuffle_moe_weight`), made on the first call
+    and kept for as long as ``w`` keeps its storage and is not written through torch (its version
+    counter).  Doubles the memory the weights take; one re-layout pass per weight tensor."""
+    key = (w.data_ptr(), tuple(w.shape), w.dtype, w.device)
+    hit = _OPERAND_ORDER_CACHE.get(key)
+    if hit is not None and hit[0] == w._version:
+        return hit[1]
+    if len(_OPERAND_ORDER_CACHE) > 256:
+        _OPERAND_ORDER_CACHE.clear()
+    sh = shuffle_moe_weight(w)
+    _OPERAND_ORDER_CACHE[key] = (w._version, sh)
+    return sh
+
 
 def get_start_end(topk_idx: torch.Tensor, sorted_idx: torch.Tensor, num_experts: int):
     """``(exp_start, exp_end)`` of each expert's run in the expert-sorted slot list
@@ -181,7 +208,8 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
                   num_experts: int = None,
                   renormalize: bool = False,
                   weights_shuffled: bool = False,
-                  alignment=None) -> torch.Tensor:
+                  alignment=None,
+                  cache_operand_order: bool = None) -> torch.Tensor:
     """fp8 MoE MLP: per-token-group quant -> gate_up grouped GEMM (+SiLU-and-mul, re-quant)
     -> down grouped GEMM (x routing weight) -> sum over the top-k slots.
 
@@ -198,6 +226,10 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     ``moe_align_block_size(topk_ids, ALIGN_BLOCK, num_experts, return_counts=True)``): the layer
     then sorts its routing once, in the router, instead of again in here (the reference sorts
     inside, fused_moe.py:314-320; that is what happens when ``alignment`` is None).
+    ``cache_operand_order=True`` (or the environment variable ``DLBLAS_HIP_CACHE_OPERAND_ORDER=1``
+    when the argument is left at None) is for callers that hand over row-major weights on every
+    call: the operand-order copies are made on the first call and reused while the weight tensors
+    stay unmodified, at the price of holding the weights twice.
     """
     _lib.require_cuda(hidden_states, w1_q, w1_s, w2_q, w2_s, topk_weights, topk_ids)
     assert hidden_states.dim() == 2 and topk_ids.shape == topk_weights.shape
@@ -208,6 +240,8 @@ def fused_moe_fp8(hidden_states: torch.Tensor,
     assert H1 == H and w2_q.shape == (E, O, I) and topk_ids.shape == (T, topk)
     assert w1_q.dtype == torch.float8_e4m3fn and w2_q.dtype == torch.float8_e4m3fn
     assert w1_q.is_contiguous() and w2_q.is_contiguous()
+    if not weights_shuffled and _cache_requested(cache_operand_order) and O % 16 == 0:
+        w1_q, w2_q, weights_shuffled = _operand_order_cached(w1_q), _operand_order_cached(w2_q), True
     assert w1_s.shape == (E, N2 // 128, H // 128) and w2_s.shape == (E, O // 128, I // 128)
     if num_experts is None:
         num_experts = E
@@ -271,14 +305,15 @@ def fused_moe(hidden_states: torch.Tensor,
               num_experts: int = None,
               renormalize: bool = False,
               weights_shuffled: bool = False,
-              alignment=None) -> torch.Tensor:
+              alignment=None,
+              cache_operand_order: bool = None) -> torch.Tensor:
     """fused moe -- signature and semantics of ``dlblas.kernels.fused_moe.fused_moe``
     (reference: fused_moe.py:296-376): ``w1`` [E, 2I, H] (gate rows first), ``w2`` [E, H, I],
     bf16/f16; routing slots are grouped by expert, the gate_up grouped GEMM runs with the
     SiLU-and-mul fused into its epilogue (same rounding points as the reference), the down
     grouped GEMM applies the routing weight and the top-k slots are summed.
-    ``weights_shuffled`` and ``alignment`` are this package's extensions (see
-    :func:`shuffle_moe_weight` and :func:`fused_moe_fp8`)."""
+    ``weights_shuffled``, ``alignment`` and ``cache_operand_order`` are this package's extensions
+    (see :func:`shuffle_moe_weight` and :func:`fused_moe_fp8`)."""
     _lib.require_cuda(hidden_states, w1, w2, topk_weights, topk_ids)
     M = hidden_states.size(0)
     E, N, _ = w1.shape
@@ -288,6 +323,8 @@ def fused_moe(hidden_states: torch.Tensor,
     assert w1.shape == (E, 2 * I, H) and w2.shape == (E, O, I)
     assert hidden_states.dtype == w1.dtype == w2.dtype
     assert w1.is_contiguous() and w2.is_contiguous()
+    if not weights_shuffled and _cache_requested(cache_operand_order) and O % 16 == 0:
+        w1, w2, weights_shuffled = _operand_order_cached(w1), _operand_order_cached(w2), True
     if num_experts is None:
         num_experts = E
     dev, dt = hidden_states.device, hidden_states.dtype

@@ -190,3 +190,25 @@ def test_sizes_that_are_not_multiples_of_128(dev, T, H, I, O, E, k, dtype):
         sh = fm.fused_moe(x.to(dev), fm.shuffle_moe_weight(w1.to(dev)), fm.shuffle_moe_weight(w2.to(dev)),
                           tw.to(dev), ids.to(dev), k, weights_shuffled=True).cpu()
         assert torch.equal(sh, out)
+
+
+def test_operand_order_cache(dev, monkeypatch):
+    # row-major weights handed over on every call, re-arranged once on the caller's behalf:
+    # same bits as the row-major path, a new copy after an in-place update of the weights
+    from dlcompiler_amd.kernels import fused_moe as fm
+
+    x, w1, w2, tw, ids = _inputs(200, 256, 128, 8, 2, 5, torch.bfloat16)
+    d = [t.to(dev) for t in (x, w1, w2, tw, ids)]
+    plain = fm.fused_moe(*d, 2)
+    fm._OPERAND_ORDER_CACHE.clear()
+    cached = fm.fused_moe(*d, 2, cache_operand_order=True)
+    assert torch.equal(cached, plain) and len(fm._OPERAND_ORDER_CACHE) == 2
+    first = fm._OPERAND_ORDER_CACHE[(d[1].data_ptr(), tuple(d[1].shape), d[1].dtype, d[1].device)][1]
+    again = fm.fused_moe(*d, 2, cache_operand_order=True)
+    assert torch.equal(again, plain)
+    assert fm._OPERAND_ORDER_CACHE[(d[1].data_ptr(), tuple(d[1].shape), d[1].dtype, d[1].device)][1] is first
+    d[1].mul_(2.0)                                            # in-place update: the copy is stale
+    upd = fm.fused_moe(*d, 2, cache_operand_order=True)
+    assert torch.equal(upd, fm.fused_moe(*d, 2)) and not torch.equal(upd, plain)
+    monkeypatch.setenv("DLBLAS_HIP_CACHE_OPERAND_ORDER", "1")  # the switch for unmodified callers
+    assert torch.equal(fm.fused_moe(*d, 2), upd)
