@@ -478,9 +478,15 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         graph_ms = _graph_replay_ms(
             lambda: fm.fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled), 20, 5, "moe " + name)
         st_gu, st_dn = kernel_times(dw, shuffled)
+        # the same step when the layer's router has already produced the expert alignment
+        # (moe_topk_softmax_align) and hands it over: the routing is sorted once per layer
+        al_sorted, _, _, al_counts = moe_align_block_size(ids, fm.ALIGN_BLOCK, E, return_counts=True)
+        ms_al, _ = _time_steps(lambda i: fm.fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled,
+                                                         alignment=(al_sorted, al_counts)), steps, warmup)
         layouts[name] = {
             "ms_per_step": ms, "value": flops / ms / 1e9, "unit": "TFLOP/s", "timing": st,
             "graph_replay_ms": graph_ms,
+            "alignment_handed_over": {"ms_per_step": ms_al, "value": flops / ms_al / 1e9, "unit": "TFLOP/s"},
             "gate_up_kernel": dict(st_gu, tflops=gate_up_flops / st_gu["median_ms"] / 1e9,
                                    frac=gate_up_flops / st_gu["median_ms"] / 1e9 / PEAK_FP8_TFLOPS),
             "down_kernel": dict(st_dn, tflops=down_flops / st_dn["median_ms"] / 1e9,

@@ -50,9 +50,12 @@ def gating():
     w_raw, _ = og.topk_softmax(logits, 6, False)
     s, e, tot, cnt = og.align_block_size(ids, 16, 64)
     start, end = og.start_end(ids, 64)
+    # the reference's fused gate kernel in its own output form (full softmax, one-hot masks)
+    gates, masks = og.topk_gating_part1(logits, 6)
+    assert torch.equal(masks.argmax(-1).t().to(torch.int32), ids)   # same selection as the index form
     fio.save("moe_gating", logits=logits, k=6, block=16, weights=w, weights_no_renorm=w_raw,
              ids=ids, sorted_token_ids=s, expert_ids=e, num_tokens_post_padded=tot, counts=cnt,
-             exp_start=start, exp_end=end)
+             exp_start=start, exp_end=end, gates=gates, masks=masks)
 
 
 def prefill():
@@ -117,8 +120,14 @@ def decoder_ops():
     w = torch.rand((256,), generator=g).to(BF)
     res = torch.randn((5, 256), generator=g).to(BF)
     out_add, res_out = odec.rms_norm(x, w, 1e-6, residual=res)
+    # a row length that is no whole number of 16-byte vectors (the element-wise kernel)
+    x77 = torch.randn((3, 77), generator=g).to(HF)
+    w77 = torch.rand((77,), generator=g).to(HF)
+    r77 = torch.randn((3, 77), generator=g).to(HF)
+    o77, ro77 = odec.rms_norm(x77, w77, 1e-6, residual=r77)
     fio.save("rms_norm", x=x, weight=w, residual=res, eps=1e-6, out=odec.rms_norm(x, w, 1e-6),
-             out_add=out_add, residual_out=res_out)
+             out_add=out_add, residual_out=res_out, x77=x77, weight77=w77, residual77=r77,
+             out77=odec.rms_norm(x77, w77, 1e-6), out_add77=o77, residual_out77=ro77)
 
     T, hq, hk, d = 6, 4, 2, 64
     q = torch.randn((T, hq, d), generator=g).to(HF)
@@ -127,7 +136,15 @@ def decoder_ops():
     cos = torch.cat((ang.cos(), ang.cos()), -1).to(HF)
     sin = torch.cat((ang.sin(), ang.sin()), -1).to(HF)
     rq, rk_ = odec.apply_rotary_pos_emb(q.float(), k.float(), cos.float(), sin.float())
-    fio.save("apply_rotary_pos_emb", q=q, k=k, cos=cos, sin=sin, q_embed_f32=rq, k_embed_f32=rk_)
+    # head size 6: not a multiple of a 16-byte vector (the element-wise kernel)
+    q6 = torch.randn((T, 3, 6), generator=g).to(BF)
+    k6 = torch.randn((T, 1, 6), generator=g).to(BF)
+    a6 = torch.rand((T, 1, 3), generator=g) * 6.28
+    c6 = torch.cat((a6.cos(), a6.cos()), -1).to(BF)
+    s6 = torch.cat((a6.sin(), a6.sin()), -1).to(BF)
+    rq6, rk6 = odec.apply_rotary_pos_emb(q6.float(), k6.float(), c6.float(), s6.float())
+    fio.save("apply_rotary_pos_emb", q=q, k=k, cos=cos, sin=sin, q_embed_f32=rq, k_embed_f32=rk_,
+             q6=q6, k6=k6, cos6=c6, sin6=s6, q6_embed_f32=rq6, k6_embed_f32=rk6)
 
 
 def moe():
@@ -148,9 +165,22 @@ def moe():
              out=ofm.fused_moe_fp8(x, w1q, w1s, w2q, w2s, tw, ids))
 
 
+def launcher():
+    # the reference's grouped-GEMM launcher case in small (test_fused_moe.py:17-145)
+    g = gen(106)
+    M, K, N, E, k = 24, 64, 16, 3, 2
+    A = ((torch.rand((M, K), generator=g) - 0.5) / 2).to(HF)
+    B = ((torch.rand((E, N, K), generator=g) - 0.5) / 2).to(HF)
+    weights, idx = torch.rand((M, E), generator=g).to(HF).topk(k, dim=-1)
+    sorted_idx = idx.flatten().argsort(stable=True)
+    start, end = og.start_end(idx, E)
+    fio.save("moe_launcher", a=A, b=B, weights=weights, topk_idx=idx, sorted_idx=sorted_idx,
+             exp_start=start, exp_end=end, top_k=k, out=ofm.grouped_gemm_launcher(A, B, idx, weights))
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
-    for make in (silu, gating, prefill, paged, decoder_ops, moe):
+    for make in (silu, gating, prefill, paged, decoder_ops, moe, launcher):
         make()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):

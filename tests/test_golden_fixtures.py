@@ -25,7 +25,8 @@ fio = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(fio)
 
 NAMES = ["silu_and_mul", "moe_gating", "prefill_attention", "paged_decode", "paged_prefill",
-         "fill_kv_cache", "rms_norm", "apply_rotary_pos_emb", "fused_moe_bf16", "fused_moe_fp8"]
+         "fill_kv_cache", "rms_norm", "apply_rotary_pos_emb", "fused_moe_bf16", "fused_moe_fp8",
+         "moe_launcher"]
 
 
 def _ulp(dtype):
@@ -70,6 +71,9 @@ def test_oracle_reproduces_gating():
     assert torch.equal(tot, f["num_tokens_post_padded"]) and torch.equal(cnt, f["counts"])
     start, end = og.start_end(f["ids"], 64)
     assert torch.equal(start, f["exp_start"]) and torch.equal(end, f["exp_end"])
+    gates, masks = og.topk_gating_part1(f["logits"], f["k"])
+    torch.testing.assert_close(gates, f["gates"], rtol=1e-6, atol=0)
+    assert torch.equal(masks, f["masks"])
 
 
 def test_oracle_reproduces_attention():
@@ -98,11 +102,19 @@ def test_oracle_reproduces_decoder_ops():
     out, res = odec.rms_norm(f["x"], f["weight"], f["eps"], residual=f["residual"])
     _same(out, f["out_add"])
     assert torch.equal(res, f["residual_out"])
+    _same(odec.rms_norm(f["x77"], f["weight77"], f["eps"]), f["out77"])
+    out, res = odec.rms_norm(f["x77"], f["weight77"], f["eps"], residual=f["residual77"])
+    _same(out, f["out_add77"])
+    assert torch.equal(res, f["residual_out77"])
     f = fio.load("apply_rotary_pos_emb")
     rq, rk = odec.apply_rotary_pos_emb(f["q"].float(), f["k"].float(), f["cos"].float(),
                                        f["sin"].float())
     _same(rq, f["q_embed_f32"])
     _same(rk, f["k_embed_f32"])
+    rq, rk = odec.apply_rotary_pos_emb(f["q6"].float(), f["k6"].float(), f["cos6"].float(),
+                                       f["sin6"].float())
+    _same(rq, f["q6_embed_f32"])
+    _same(rk, f["k6_embed_f32"])
 
 
 def test_oracle_reproduces_moe():
@@ -114,6 +126,10 @@ def test_oracle_reproduces_moe():
     assert torch.equal(s, f["hidden_scale"])
     _same(ofm.fused_moe_fp8(f["hidden"], f["w1_q"], f["w1_s"], f["w2_q"], f["w2_s"],
                             f["topk_weights"], f["topk_ids"]), f["out"])
+    f = fio.load("moe_launcher")
+    _same(ofm.grouped_gemm_launcher(f["a"], f["b"], f["topk_idx"], f["weights"]), f["out"])
+    start, end = og.start_end(f["topk_idx"], f["b"].shape[0])
+    assert torch.equal(start, f["exp_start"]) and torch.equal(end, f["exp_end"])
 
 
 # ------------------------------------------------------------------ GPU: HIP path vs fixtures
@@ -154,6 +170,11 @@ def test_hip_gating_matches_fixture(dev):
     assert torch.equal(cnt.cpu(), f["counts"]) and torch.equal(fused[1].cpu(), f["ids"])
     start, end = get_start_end(ids, torch.empty(0, dtype=torch.int64, device=dev), 64)
     assert torch.equal(start.cpu(), f["exp_start"]) and torch.equal(end.cpu(), f["exp_end"])
+    from dlcompiler_amd.kernels.topk_gating_fwd_part1 import call as gating_part1
+
+    gates, masks = gating_part1(logits, f["k"])
+    torch.testing.assert_close(gates.cpu(), f["gates"], rtol=2e-6, atol=0)
+    assert torch.equal(masks.cpu(), f["masks"])
 
 
 @pytest.mark.gpu
@@ -207,11 +228,20 @@ def test_hip_decoder_ops_match_fixtures(dev):
     out, res = rms_norm(f["x"].to(dev), f["weight"].to(dev), f["eps"], residual=f["residual"].to(dev))
     assert torch.equal(res.cpu(), f["residual_out"])
     torch.testing.assert_close(out.cpu(), f["out_add"], **tol)
+    tol77 = dict(rtol=2e-3, atol=1e-5)                      # fp16 rows of 77 elements
+    torch.testing.assert_close(rms_norm(f["x77"].to(dev), f["weight77"].to(dev), f["eps"]).cpu(),
+                               f["out77"], **tol77)
+    out, res = rms_norm(f["x77"].to(dev), f["weight77"].to(dev), f["eps"], residual=f["residual77"].to(dev))
+    assert torch.equal(res.cpu(), f["residual_out77"])
+    torch.testing.assert_close(out.cpu(), f["out_add77"], **tol77)
 
     f = fio.load("apply_rotary_pos_emb")
     qe, ke = apply_rotary_pos_emb(f["q"].to(dev), f["k"].to(dev), f["cos"].to(dev), f["sin"].to(dev))
     torch.testing.assert_close(qe.cpu().float(), f["q_embed_f32"], rtol=1e-5, atol=2e-3)
     torch.testing.assert_close(ke.cpu().float(), f["k_embed_f32"], rtol=1e-5, atol=2e-3)
+    qe, ke = apply_rotary_pos_emb(f["q6"].to(dev), f["k6"].to(dev), f["cos6"].to(dev), f["sin6"].to(dev))
+    torch.testing.assert_close(qe.cpu().float(), f["q6_embed_f32"], rtol=1.6e-2, atol=1e-2)
+    torch.testing.assert_close(ke.cpu().float(), f["k6_embed_f32"], rtol=1.6e-2, atol=1e-2)
 
 
 @pytest.mark.gpu
@@ -231,3 +261,12 @@ def test_hip_moe_matches_fixtures(dev):
                         f["w2_s"].to(dev), f["topk_weights"].to(dev), f["topk_ids"].to(dev), f["topk"])
     ref = f["out"].double()
     assert ((out.cpu().double() - ref).norm() / ref.norm()).item() <= 3e-2
+
+    from dlcompiler_amd.kernels.fused_moe import fused_moe_kernel_launcher
+
+    f = fio.load("moe_launcher")
+    C = torch.zeros(f["out"].shape, dtype=f["out"].dtype, device=dev)
+    fused_moe_kernel_launcher(f["a"].to(dev), f["b"].to(dev), C, f["sorted_idx"].to(dev),
+                              f["exp_start"].to(dev), f["exp_end"].to(dev), f["weights"].to(dev),
+                              enable_weights=True, top_k=f["top_k"], num_tokens=f["a"].shape[0])
+    torch.testing.assert_close(C.cpu(), f["out"])
