@@ -804,7 +804,7 @@ def load_probe_lib():
         lib.dlb_probe_mfma_operand_bytes.restype = c_int64
         lib.dlb_probe_mfma_operand_bytes.argtypes = [c_int]
         lib.dlb_probe_mfma_rate.restype = c_int
-        lib.dlb_probe_mfma_rate.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int,
+        lib.dlb_probe_mfma_rate.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int,
                                             c_void_p]
         lib.dlb_probe_hbm_read.restype = c_int
         lib.dlb_probe_hbm_read.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p]
@@ -834,13 +834,13 @@ def measure_box(dev):
         "fp8_zeros": torch.zeros(nbytes, dtype=torch.uint8, device=dev),
     }
     out = {}
-    for key, buf in operands.items():
-        fp8 = int(key.startswith("fp8"))
+
+    def mfma_rate(buf, fp8, valu):
         iters = 20000 if fp8 else 40000   # about 12 ms per launch on random operands
 
         def launch():
             _lib.check(lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sink_bytes,
-                                               blocks, fp8, iters, stream), "dlb_probe_mfma_rate")
+                                               blocks, fp8, iters, valu, stream), "dlb_probe_mfma_rate")
 
         for _ in range(3):
             launch()
@@ -851,8 +851,16 @@ def measure_box(dev):
             launch()
         t.stop(ev)
         ms = t.mean_ms() / 3
-        flops = blocks * 8 * iters * 4 * (131072 if fp8 else 32768)
-        out[f"mfma_{key}_tflops"] = flops / ms / 1e9
+        return blocks * 8 * iters * 4 * (131072 if fp8 else 32768) / ms / 1e9
+
+    for key, buf in operands.items():
+        out[f"mfma_{key}_tflops"] = mfma_rate(buf, int(key.startswith("fp8")), 0)
+    # the same stream with 8 independent fp32 multiply-adds of the wave behind every MFMA: what
+    # the SIMD hides of a wave's vector arithmetic under its matrix instructions (the prefill
+    # kernel issues about 5 vector instructions per bf16 MFMA, 32 of them exponentials per tile;
+    # the fp8 GEMM's main loop about 10 per MFMA, 8 of them the block-scale multiplies)
+    out["mfma_bf16_randn_valu8_tflops"] = mfma_rate(operands["bf16_randn"], 0, 8)
+    out["mfma_fp8_randn_valu8_tflops"] = mfma_rate(operands["fp8_randn"], 1, 8)
     x = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()   # 1 GiB
     nb = x.numel() * 4
 
@@ -871,7 +879,8 @@ def measure_box(dev):
     out["hbm_read_gbs"] = nb / (t.mean_ms() / 10) / 1e6
     out["note"] = ("measured in this run: back-to-back MFMAs (bf16 32x32x16 / fp8 32x32x64, two waves "
                    "per SIMD on every CU, nothing else in the loop) on random-normal and on all-zero "
-                   "operands; a read-only non-temporal stream over 1 GiB")
+                   "operands; valu8: the same with 8 independent fp32 multiply-adds of the wave after "
+                   "every MFMA; a read-only non-temporal stream over 1 GiB")
     del x
     torch.cuda.empty_cache()
     return out
@@ -945,10 +954,12 @@ def main():
         torch.cuda.empty_cache()
     box = None if args.counters else measure_box(dev)
     if box is not None:
-        print("[bench] this chip, measured: MFMA bf16 %.0f TFLOP/s on random operands (%.0f on zeros), "
-              "fp8 %.0f (%.0f), read-only HBM stream %.0f GB/s" % (
+        print("[bench] this chip, measured: MFMA bf16 %.0f TFLOP/s on random operands (%.0f on zeros, %.0f "
+              "with 8 vector multiply-adds per MFMA), fp8 %.0f (%.0f, %.0f), read-only HBM stream %.0f GB/s" % (
                   box["mfma_bf16_randn_tflops"], box["mfma_bf16_zeros_tflops"],
-                  box["mfma_fp8_randn_tflops"], box["mfma_fp8_zeros_tflops"], box["hbm_read_gbs"]),
+                  box["mfma_bf16_randn_valu8_tflops"],
+                  box["mfma_fp8_randn_tflops"], box["mfma_fp8_zeros_tflops"],
+                  box["mfma_fp8_randn_valu8_tflops"], box["hbm_read_gbs"]),
               file=sys.stderr, flush=True)
     names = list(WORKLOADS) if args.workload == "all" else [args.workload]
     primary = PRIMARY if args.workload == "all" else args.workload

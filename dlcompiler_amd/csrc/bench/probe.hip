@@ -6,7 +6,9 @@
 //
 // Every wave cycles through four operand pairs read once from `operands` (so the registers hold
 // the caller's data, whatever its entropy) and issues `iters` rounds of four independent MFMAs;
-// no memory traffic, LDS or vector arithmetic inside the loop.
+// no memory traffic or LDS inside the loop, and vector arithmetic only on request: with
+// valu_per_mfma > 0 it measures how much of a wave's vector work the SIMD hides under its
+// matrix instructions.
 #include "../common.h"
 #include "bench_probe.h"
 
@@ -16,7 +18,10 @@ namespace {
 constexpr int kProbeThreads = 512;      // two waves per SIMD
 constexpr int kProbeWordsPerLane = 64;  // 4 pairs x (two 16-byte halves of A and of B)
 
-template <bool FP8>
+// NV > 0: every MFMA is followed by NV independent fp32 multiply-adds of the same wave (eight
+// dependency chains), the mix of a kernel that does vector arithmetic between its matrix
+// instructions; a scheduling fence after each group keeps the two kinds interleaved as written.
+template <bool FP8, int NV>
 __global__ __launch_bounds__(kProbeThreads) void mfma_rate_kernel(const uint32_t* __restrict__ data,
                                                                   float* sink, int iters) {
   u32x4 a[4], b[4], a2[4], b2[4];
@@ -33,6 +38,10 @@ __global__ __launch_bounds__(kProbeThreads) void mfma_rate_kernel(const uint32_t
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  float x[8];
+#pragma unroll
+  for (int f = 0; f < 8; ++f) x[f] = 1.0f + 0.001f * (float)((threadIdx.x + f) & 7);
+  const float c1 = 1.0f - 1e-6f * (float)(iters & 1), c2 = 1e-6f * (float)(iters & 3);
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -47,9 +56,16 @@ __global__ __launch_bounds__(kProbeThreads) void mfma_rate_kernel(const uint32_t
                                                          __builtin_bit_cast(bf16x8, b[i]), acc[i],
                                                          0, 0, 0);
       }
+      if (NV > 0) {
+#pragma unroll
+        for (int f = 0; f < NV; ++f) x[f & 7] = __builtin_fmaf(x[f & 7], c1, c2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   float s = 0.0f;
+#pragma unroll
+  for (int f = 0; f < 8; ++f) s += x[f];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -100,18 +116,28 @@ extern "C" int64_t dlb_probe_mfma_operand_bytes(int blocks) {
 
 extern "C" int dlb_probe_mfma_rate(const void* operands, int64_t operand_bytes, void* sink,
                                    int64_t sink_bytes, int blocks, int fp8, int iters,
-                                   void* stream) {
+                                   int valu_per_mfma, void* stream) {
   using namespace dlb;
   if (blocks < 1 || iters < 0 || !operands || !sink) return DLB_ERR_BAD_ARG;
+  if (valu_per_mfma != 0 && valu_per_mfma != 4 && valu_per_mfma != 8 && valu_per_mfma != 16)
+    return DLB_ERR_UNSUPPORTED;
   if (sink_bytes < DLB_PROBE_SINK_BYTES) return DLB_ERR_WORKSPACE;
   if (operand_bytes < dlb_probe_mfma_operand_bytes(blocks)) return DLB_ERR_WORKSPACE;
   if (!aligned16(operands)) return DLB_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
-  if (fp8)
-    hipLaunchKernelGGL(mfma_rate_kernel<true>, dim3((uint32_t)blocks), dim3(kProbeThreads), 0, s,
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(kProbeThreads), 0, s,
                        (const uint32_t*)operands, (float*)sink, iters);
-  else
-    hipLaunchKernelGGL(mfma_rate_kernel<false>, dim3((uint32_t)blocks), dim3(kProbeThreads), 0, s,
-                       (const uint32_t*)operands, (float*)sink, iters);
+  };
+  switch (valu_per_mfma + (fp8 ? 100 : 0)) {
+    case 0: launch(mfma_rate_kernel<false, 0>); break;
+    case 4: launch(mfma_rate_kernel<false, 4>); break;
+    case 8: launch(mfma_rate_kernel<false, 8>); break;
+    case 16: launch(mfma_rate_kernel<false, 16>); break;
+    case 100: launch(mfma_rate_kernel<true, 0>); break;
+    case 104: launch(mfma_rate_kernel<true, 4>); break;
+    case 108: launch(mfma_rate_kernel<true, 8>); break;
+    default: launch(mfma_rate_kernel<true, 16>); break;
+  }
   return launch_status();
 }

@@ -19,10 +19,13 @@ def test_probes_launch_and_check_arguments(dev):
     assert nbytes == blocks * 512 * 256
     buf = torch.randn(nbytes // 2, device=dev).bfloat16()
     for fp8 in (0, 1):
-        assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sb, blocks, fp8, 10, stream) == 0
-    assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes - 16, sink.data_ptr(), sb, blocks, 0, 10, stream) == -4
-    assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sb - 4, blocks, 0, 10, stream) == -4
-    assert lib.dlb_probe_mfma_rate(None, nbytes, sink.data_ptr(), sb, blocks, 0, 10, stream) == -1
+        for valu in (0, 4, 8, 16):
+            assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sb, blocks, fp8, 10, valu,
+                                           stream) == 0
+    assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sb, blocks, 0, 10, 5, stream) == -2
+    assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes - 16, sink.data_ptr(), sb, blocks, 0, 10, 0, stream) == -4
+    assert lib.dlb_probe_mfma_rate(buf.data_ptr(), nbytes, sink.data_ptr(), sb - 4, blocks, 0, 10, 0, stream) == -4
+    assert lib.dlb_probe_mfma_rate(None, nbytes, sink.data_ptr(), sb, blocks, 0, 10, 0, stream) == -1
     assert lib.dlb_probe_hbm_read(buf.data_ptr(), sink.data_ptr(), sb, nbytes, stream) == 0
     assert lib.dlb_probe_hbm_read(buf.data_ptr(), sink.data_ptr(), sb, 24, stream) == -2
     assert lib.dlb_probe_hbm_read(buf.data_ptr(), sink.data_ptr(), 64, nbytes, stream) == -4
