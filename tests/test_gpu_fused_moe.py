@@ -212,3 +212,36 @@ def test_operand_order_cache(dev, monkeypatch):
     assert torch.equal(upd, fm.fused_moe(*d, 2)) and not torch.equal(upd, plain)
     monkeypatch.setenv("DLBLAS_HIP_CACHE_OPERAND_ORDER", "1")  # the switch for unmodified callers
     assert torch.equal(fm.fused_moe(*d, 2), upd)
+
+
+def test_zero_tokens(dev):
+    """Empty batches (a decode step in which no token is routed to this rank) go through every MoE
+    entry point and come back as empty results of the right shape."""
+    from dlcompiler_amd.kernels import topk_gating_fwd_part1
+    from dlcompiler_amd.kernels.fused_moe import (fused_moe, fused_moe_fp8,
+                                                  fused_moe_kernel_launcher)
+    from dlcompiler_amd.kernels.moe_gating import moe_topk_softmax_align
+
+    E, H, I, k = 8, 256, 128, 2
+    x = torch.empty((0, H), dtype=torch.bfloat16, device=dev)
+    w1 = torch.zeros((E, 2 * I, H), dtype=torch.bfloat16, device=dev)
+    w2 = torch.zeros((E, H, I), dtype=torch.bfloat16, device=dev)
+    tw = torch.empty((0, k), device=dev)
+    ids = torch.empty((0, k), dtype=torch.int32, device=dev)
+    assert fused_moe(x, w1, w2, tw, ids, k).shape == (0, H)
+    w1s = torch.ones((E, 2 * I // 128, H // 128), device=dev)
+    w2s = torch.ones((E, H // 128, I // 128), device=dev)
+    out = fused_moe_fp8(x, w1.to(torch.float8_e4m3fn), w1s, w2.to(torch.float8_e4m3fn), w2s, tw, ids, k)
+    assert out.shape == (0, H) and out.dtype == torch.bfloat16
+    gates, masks = topk_gating_fwd_part1.call(torch.empty((0, E), device=dev), k)
+    assert gates.shape == (0, E) and masks.shape == (k, 0, E)
+    w, i, sorted_ids, expert_ids, npad, counts = moe_topk_softmax_align(
+        torch.empty((0, E), device=dev), k, 128, return_counts=True)
+    assert w.shape == (0, k) and int(npad.item()) == 0 and (counts == 0).all() and (expert_ids == -1).all()
+    C = torch.empty((0, 128), dtype=torch.bfloat16, device=dev)
+    none = torch.zeros((4,), dtype=torch.int64, device=dev)
+    fused_moe_kernel_launcher(torch.empty((0, 64), dtype=torch.bfloat16, device=dev),
+                              torch.zeros((4, 128, 64), dtype=torch.bfloat16, device=dev), C,
+                              torch.empty((0,), dtype=torch.int64, device=dev), none, none, None,
+                              False, 2, 0, 0, True, True)
+    torch.cuda.synchronize()
