@@ -418,7 +418,7 @@ def wl_decode(dev, steps, warmup, cpu):
 def wl_moe_fp8(dev, steps, warmup, cpu):
     from dlcompiler_amd import _lib
     from dlcompiler_amd.kernels import fused_moe as fm
-    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size, moe_topk_softmax_align
     from oracle import fp8 as ofp8
     from oracle import moe_gating as og
 
@@ -483,10 +483,22 @@ def wl_moe_fp8(dev, steps, warmup, cpu):
         al_sorted, _, _, al_counts = moe_align_block_size(ids, fm.ALIGN_BLOCK, E, return_counts=True)
         ms_al, _ = _time_steps(lambda i: fm.fused_moe_fp8(x, *dw, tw, ids, K, weights_shuffled=shuffled,
                                                          alignment=(al_sorted, al_counts)), steps, warmup)
+        # and the whole layer from the router's logits: softmax + top-k + alignment (one native call
+        # of two launches), then the MLP on the alignment that call returns
+        logits_dev = logits.to(dev)
+
+        def from_logits(i):
+            w_, ids_, so_, _, _, cn_ = moe_topk_softmax_align(logits_dev, K, fm.ALIGN_BLOCK,
+                                                                 return_counts=True)
+            fm.fused_moe_fp8(x, *dw, w_, ids_, K, weights_shuffled=shuffled, alignment=(so_, cn_))
+
+        ms_fl, _ = _time_steps(from_logits, steps, warmup)
         layouts[name] = {
             "ms_per_step": ms, "value": flops / ms / 1e9, "unit": "TFLOP/s", "timing": st,
             "graph_replay_ms": graph_ms,
             "alignment_handed_over": {"ms_per_step": ms_al, "value": flops / ms_al / 1e9, "unit": "TFLOP/s"},
+            "from_router_logits": {"ms_per_step": ms_fl, "value": flops / ms_fl / 1e9, "unit": "TFLOP/s",
+                                   "note": "router softmax + top-k + alignment included in the step"},
             "gate_up_kernel": dict(st_gu, tflops=gate_up_flops / st_gu["median_ms"] / 1e9,
                                    frac=gate_up_flops / st_gu["median_ms"] / 1e9 / PEAK_FP8_TFLOPS),
             "down_kernel": dict(st_dn, tflops=down_flops / st_dn["median_ms"] / 1e9,
