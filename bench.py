@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
-Runs the five BASELINE.json configurations (fused silu_and_mul, MoE gating + alignment,
+Runs the five benchmark configurations (fused silu_and_mul, MoE gating + alignment,
 varlen causal prefill attention, paged decode attention, fp8 fused-MoE MLP), the reference's own
 bf16 fused_moe at the config-5 shape and four neighbouring decoder-layer operators (add + RMSNorm,
 rotary embedding, KV-cache fill, paged prefill) on synthetic,

@@ -81,7 +81,7 @@ def test_special_values(dev):
 
 
 def test_config_shape_full(dev):
-    # BASELINE config 1: bf16 [8192, 2 x 11008] ~ N(0,1), seed 0
+    # benchmark configuration 1: bf16 [8192, 2 x 11008] ~ N(0,1), seed 0
     g = torch.Generator().manual_seed(0)
     x = torch.randn((8192, 22016), generator=g).bfloat16()
     out = _run(x, dev)

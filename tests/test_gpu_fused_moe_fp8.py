@@ -148,7 +148,7 @@ def test_deterministic(dev):
 
 
 def test_config5_full(dev):
-    """BASELINE config 5: 4096 tokens, hidden 2048, intermediate 1408, 64 experts, top-6."""
+    """benchmark configuration 5: 4096 tokens, hidden 2048, intermediate 1408, 64 experts, top-6."""
     from dlcompiler_amd.kernels.fused_moe import fused_moe_fp8
 
     T, H, I, E, k = 4096, 2048, 1408, 64, 6

@@ -141,7 +141,7 @@ def test_align_is_deterministic(dev):
 
 
 def test_end_to_end_config2(dev):
-    # BASELINE config 2: logits fp32 [16384, 64] ~ N(0,1) seed 1, k = 6, block 64
+    # benchmark configuration 2: logits fp32 [16384, 64] ~ N(0,1) seed 1, k = 6, block 64
     from dlcompiler_amd.kernels.moe_gating import moe_align_block_size, moe_topk_softmax
 
     g = torch.Generator().manual_seed(1)

@@ -159,7 +159,7 @@ def test_unsupported_requests_raise(dev):
 
 
 def test_config4_full(dev):
-    """BASELINE config 4: batch 64, ctx uniform in [512, 8192] (seed 3), 64-token pages,
+    """benchmark configuration 4: batch 64, ctx uniform in [512, 8192] (seed 3), 64-token pages,
     32 query / 8 KV heads, head_dim 128, bf16; block table [64, 128] from a seeded permutation."""
     from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
 
