@@ -133,9 +133,20 @@ def torch_dtype_code(dtype) -> int:
     return table[dtype]
 
 
+_raw_stream = None
+
+
 def current_stream_ptr(device) -> int:
+    """The ``hipStream_t`` of torch's current stream on ``device``, as an integer."""
+    global _raw_stream
     import torch
 
+    if _raw_stream is None:
+        # the raw accessor costs a sixth of building a torch.cuda.Stream object per launch
+        _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", False)
+    if _raw_stream:
+        index = device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(device).cuda_stream
 
 

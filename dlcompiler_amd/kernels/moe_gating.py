@@ -138,17 +138,19 @@ def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_ex
     plan = _FUSED_PLANS.get((T, E, k, block_size))
     if plan is None:
         ws_words = max((lib.dlb_moe_topk_softmax_align_ws_bytes(T, E) + 3) // 4, 1)
-        # one allocation of 4-byte words, carved into the results and the scratch (each piece
-        # followed by the padding that keeps the next one 16-byte aligned)
-        pieces = []
-        for n in (numel, numel, cap, nblk, 1, ws_words, E):
-            pieces += [n, -n & 3]
+        # one allocation of 4-byte words, carved into the results and the scratch; every piece
+        # is rounded up to 16 bytes so that the next one starts aligned, and a piece that was
+        # rounded is trimmed afterwards (the one-word total goes last and needs neither)
+        sizes = (numel, numel, cap, nblk, ws_words, E, 1)
+        pieces = [n + (-n & 3) for n in sizes[:-1]] + [1]
         if len(_FUSED_PLANS) > 64:
             _FUSED_PLANS.clear()
-        plan = _FUSED_PLANS[(T, E, k, block_size)] = (pieces, sum(pieces))
-    pieces, total = plan
+        trims = tuple(None if n == p else n for n, p in zip(sizes, pieces))
+        plan = _FUSED_PLANS[(T, E, k, block_size)] = (trims, pieces, sum(pieces))
+    trims, pieces, total = plan
     buf = torch.empty((total,), dtype=torch.int32, device=dev)
-    w_raw, _, ids, _, sorted_ids, _, expert_ids, _, num_post, _, ws, _, counts, _ = buf.split(pieces)
+    parts = [t if n is None else t.narrow(0, 0, n) for t, n in zip(buf.split(pieces), trims)]
+    w_raw, ids, sorted_ids, expert_ids, ws, counts, num_post = parts
     weights = w_raw.view(torch.float32).view(T, k)
     ids = ids.view(T, k)
     with _lib.device_guard(dev):
