@@ -125,6 +125,15 @@ def test_small_pages(dev, page):
     _run_case(dev, [65, 5], [130, 3], 2, 1, 64, page, torch.float16, seed=page + 1, window=40)
 
 
+# pages that hold several whole 64-key tiles (a power of two and not): the page of a tile is one
+# look-up and the tile starts at a slot that is a multiple of 64 inside it
+@pytest.mark.parametrize("page", [128, 192, 256])
+def test_pages_of_several_tiles(dev, page):
+    _run_case(dev, [70, 33, 129, 1, 300], [45, 0, 200, 700, 1000], 4, 2, 128, page, torch.bfloat16, seed=page)
+    _run_case(dev, [65, 130], [130, 500], 2, 1, 64, page, torch.float16, seed=page + 1, window=150)
+    _run_case(dev, [64, 128], [64, 256], 8, 2, 128, page, torch.bfloat16, seed=page + 2, softcap=25.0)
+
+
 # the index tensors are read in the integer width they arrive in: all int32, all int64 (what
 # lmdeploy hands over), mixtures, and a narrower type that the wrapper converts
 @pytest.mark.parametrize("idx", [(torch.int32,) * 4, (torch.int64,) * 4,
