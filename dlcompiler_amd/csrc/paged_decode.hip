@@ -484,8 +484,8 @@ int pick_num_teams(int units_per_team) {
 
 extern "C" size_t dlb_paged_decode_ws_bytes(int B, int Hq, int Hkv, int D, int page,
                                             int max_blocks) {
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || D > 128 || page <= 0 || max_blocks <= 0) return 0;
-  D = D <= 64 ? 64 : 128;  // the head size the kernels are built for
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || D > 256 || page <= 0 || max_blocks <= 0) return 0;
+  D = D <= 64 ? 64 : D <= 128 ? 128 : 256;  // the head size the kernels are built for
   const int group = Hq / Hkv;
   const int hchunks = (group + 15) / 16;
   const int64_t max_ctx = (int64_t)page * max_blocks;
@@ -509,9 +509,11 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
   if (Hq % Hkv != 0) return DLB_ERR_BAD_ARG;
   if (B == 0) return DLB_OK;
   if (!q || !k_cache || !v_cache || !o || !block_table || !kv_len) return DLB_ERR_BAD_ARG;
-  if (D % 8 != 0 || Dv % 8 != 0 || D > 128 || Dv > 128) return DLB_ERR_UNSUPPORTED;
-  const int Dp = (D <= 64 && Dv <= 64) ? 64 : 128;  // head size the kernel instance is built for
-  const bool ragged = D != Dp || Dv != Dp;
+  if (D % 8 != 0 || Dv % 8 != 0 || D > 256 || Dv > 256) return DLB_ERR_UNSUPPORTED;
+  // head size the kernel instance is built for; past 128 one instance, for 256, takes every size
+  // on its ragged path
+  const int Dp = (D <= 64 && Dv <= 64) ? 64 : (D <= 128 && Dv <= 128) ? 128 : 256;
+  const bool ragged = D != Dp || Dv != Dp || Dp == 256;
   if (page % 16 != 0) return DLB_ERR_UNSUPPORTED;
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
   if ((int64_t)page * max_blocks > 0x7fffffff) return DLB_ERR_UNSUPPORTED;
@@ -588,13 +590,22 @@ extern "C" int dlb_paged_decode_attn(const void* q, const void* k_cache, const v
     }                                                                                     \
     hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, D_>), grid2, dim3(D_), 0, s, p); \
   } while (0)
+#define DLB_LAUNCH_DECODE_256(DT_)                                                         \
+  do {                                                                                    \
+    if (p.page_shift >= 0) DLB_LAUNCH_SPLIT(DT_, 256, true, true);                        \
+    else DLB_LAUNCH_SPLIT(DT_, 256, false, true);                                         \
+    hipLaunchKernelGGL((paged_decode_combine_kernel<DT_, 256>), grid2, dim3(256), 0, s, p); \
+  } while (0)
   if (dtype == DLB_DTYPE_BF16) {
-    if (Dp == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 128);
+    if (Dp == 256) DLB_LAUNCH_DECODE_256(DLB_DTYPE_BF16);
+    else if (Dp == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 128);
     else DLB_LAUNCH_DECODE(DLB_DTYPE_BF16, 64);
   } else {
-    if (Dp == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
+    if (Dp == 256) DLB_LAUNCH_DECODE_256(DLB_DTYPE_F16);
+    else if (Dp == 128) DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 128);
     else DLB_LAUNCH_DECODE(DLB_DTYPE_F16, 64);
   }
+#undef DLB_LAUNCH_DECODE_256
 #undef DLB_LAUNCH_SPLIT
 #undef DLB_LAUNCH_DECODE
   return launch_status();

@@ -102,7 +102,7 @@ struct Smem {
 // number is one wave-uniform look-up and the copies are addressed as in the packed layout (a
 // scalar base per tile plus constant lane offsets).
 template <int DT, int D, int PAGED, bool RAGGED>
-__global__ __launch_bounds__(kThreads, 2) void prefill_attn_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(kThreads, D > 128 ? 1 : 2) void prefill_attn_kernel(const PrefillParams p) {
   constexpr int KS = D / 16;  // MFMA k-steps over the head dim for S^T
   constexpr int MT = D / 32;  // 32-row tiles of O^T
   constexpr int DG = D / 8;
@@ -515,9 +515,12 @@ namespace {
 // filled in (or zeroed) by the caller.
 int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk, int Dv, int max_len,
                    float sm_scale, int dtype, void* stream) {
-  if (Dk % 8 != 0 || Dv % 8 != 0 || Dk > 128 || Dv > 128) return DLB_ERR_UNSUPPORTED;
-  const int D = (Dk <= 64 && Dv <= 64) ? 64 : 128;  // head size the kernel instance is built for
-  const bool ragged = Dk != D || Dv != D;
+  if (Dk % 8 != 0 || Dv % 8 != 0 || Dk > 256 || Dv > 256) return DLB_ERR_UNSUPPORTED;
+  // head size the kernel instance is built for; past 128 there is one instance, for 256, that
+  // takes every size on its ragged path (one workgroup per CU, one wave per SIMD: the 128 output
+  // accumulators and the 64 query registers of a lane leave no room for a second wave)
+  const int D = (Dk <= 64 && Dv <= 64) ? 64 : (Dk <= 128 && Dv <= 128) ? 128 : 256;
+  const bool ragged = Dk != D || Dv != D || D == 256;
   p.dk = Dk;
   p.dv = Dv;
   if (dtype != DLB_DTYPE_BF16 && dtype != DLB_DTYPE_F16) return DLB_ERR_UNSUPPORTED;
@@ -552,13 +555,19 @@ int launch_prefill(PrefillParams& p, bool paged, int B, int Hq, int Hkv, int Dk,
     else                                                                                          \
       hipLaunchKernelGGL((prefill_attn_kernel<DT_, D_, PG_, false>), grid, dim3(kThreads), 0, s, p); \
   } while (0)
-#define DLB_DISPATCH_PREFILL(PG_)                              \
-  if (dtype == DLB_DTYPE_BF16) {                               \
-    if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 128, PG_); \
-    else DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 64, PG_);           \
-  } else {                                                     \
-    if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 128, PG_);  \
-    else DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 64, PG_);            \
+#define DLB_DISPATCH_PREFILL(PG_)                                                                \
+  if (dtype == DLB_DTYPE_BF16) {                                                                 \
+    if (D == 256)                                                                                \
+      hipLaunchKernelGGL((prefill_attn_kernel<DLB_DTYPE_BF16, 256, PG_, true>), grid,            \
+                         dim3(kThreads), 0, s, p);                                               \
+    else if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 128, PG_);                              \
+    else DLB_LAUNCH_PREFILL(DLB_DTYPE_BF16, 64, PG_);                                             \
+  } else {                                                                                       \
+    if (D == 256)                                                                                \
+      hipLaunchKernelGGL((prefill_attn_kernel<DLB_DTYPE_F16, 256, PG_, true>), grid,             \
+                         dim3(kThreads), 0, s, p);                                               \
+    else if (D == 128) DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 128, PG_);                               \
+    else DLB_LAUNCH_PREFILL(DLB_DTYPE_F16, 64, PG_);                                              \
   }
   // pages that hold whole 64-key tiles take the kernel with one page look-up per tile (the lane
   // offsets inside a page are 32-bit)

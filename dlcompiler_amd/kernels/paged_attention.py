@@ -26,7 +26,7 @@ def paged_attention_fwd(
 
     Args follow the reference: ``q`` [tokens, Hq, D]; ``k``/``v`` caches
     [pages, page_size, Hkv, D] / [pages, page_size, Hkv, Dv] (head sizes: multiples of 8 up to
-    128, the value size may differ from the key size; ``o`` is [tokens, Hq, Dv]); ``block_offsets`` [batch, max_blocks] maps a sequence's
+    256, the value size may differ from the key size; ``o`` is [tokens, Hq, Dv]); ``block_offsets`` [batch, max_blocks] maps a sequence's
     logical pages to physical ones; ``kv_seqlens`` [batch] context lengths.  One query token
     per sequence (``q.shape[-3] == q_seqlens.size(0)``, paged_attention.py:559) takes the
     split-KV decode kernel; anything else is the prefill-with-history case
@@ -45,8 +45,8 @@ def paged_attention_fwd(
         sm_scale = 1.0 / (Lq**0.5)
     batch, head = q_seqlens.shape[0], q.shape[-2]
     is_decoding = q.shape[-3] == q_seqlens.size(0)
-    if Lk % 8 != 0 or Lv % 8 != 0 or Lk > 128 or Lv > 128:
-        raise NotImplementedError("head sizes must be multiples of 8, at most 128")
+    if Lk % 8 != 0 or Lv % 8 != 0 or Lk > 256 or Lv > 256:
+        raise NotImplementedError("head sizes must be multiples of 8, at most 256")
     assert k.dim() == 4 and v.dim() == 4 and k.shape[:3] == v.shape[:3]
     assert q.dtype == k.dtype == v.dtype == o.dtype
     num_kv_heads = k.shape[-2]

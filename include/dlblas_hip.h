@@ -171,9 +171,9 @@ int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t*
  * paged_attention.py:163-167,191-199); logit_softcapping > 0 replaces the scaled logits by
  * cap * tanh(logits / cap) (:186-189); pass <= 0 to disable either.
  * Supported: dtype bf16/f16, key head size D and value head size Dv any multiples of 8 up to
- * 128 (64 and 128 run the unmasked kernels; other sizes are computed in the next of those two
- * with the extra dims masked, as the reference splits them into power-of-two blocks,
- * kernels/paged_attention.py:531-539), page % 16 == 0, all strides multiples of 8 and base
+ * 256 (64 and 128 run the unmasked kernels; other sizes are computed in the next of 64, 128 and
+ * 256 with the extra dims masked, as the reference splits them into power-of-two blocks,
+ * kernels/paged_attention.py:531-539; sizes above 128 run one wavefront per SIMD), page % 16 == 0, all strides multiples of 8 and base
  * pointers 16-byte aligned.  ws: dlb_paged_decode_ws_bytes(B, Hq, Hkv, max(D, Dv), page,
  * max_blocks) bytes of device scratch (split-KV partials), caller-owned.
  * ---------------------------------------------------------------------------------------- */
@@ -199,8 +199,8 @@ int dlb_paged_decode_attn(const void* q, const void* k_cache, const void* v_cach
  * o[t, h] = sum_{t' <= t, same sequence} softmax_t'(q[t, h] . k[t', h / (Hq/Hkv)] * sm_scale)
  *           v[t', h / (Hq/Hkv)], softmax in fp32, P rounded to `dtype` before P.V.
  * (The reference fixes sm_scale = 1/sqrt(D); pass that for drop-in behaviour.)
- * Supported: dtype bf16/f16, D any multiple of 8 up to 128 (the reference asserts
- * D in {16, 32, 64, 128}, prefill_attention.py:160), q/k/v strides multiples of 8 and bases
+ * Supported: dtype bf16/f16, D any multiple of 8 up to 256 (the reference asserts
+ * D in {16, 32, 64, 128}, prefill_attention.py:160; sizes above 128 run one wavefront per SIMD), q/k/v strides multiples of 8 and bases
  * 16-byte aligned, o strides multiples of 4 and base 8-byte aligned.  Tokens outside every
  * sequence are not written.
  * ---------------------------------------------------------------------------------------- */
@@ -225,7 +225,7 @@ int dlb_prefill_attn_varlen(const void* q, const void* k, const void* v, void* o
  *   keys >= position - window_size (:429-431,457-458); logit_softcapping > 0 replaces the
  *   scaled logits by cap * tanh(logits / cap) (:450-453).  Pass <= 0 to disable either.
  *   max_q_len >= max(q_len) sizes the grid.
- * Supported: dtype bf16/f16, D and Dv any multiples of 8 up to 128 (as for the decode entry
+ * Supported: dtype bf16/f16, D and Dv any multiples of 8 up to 256 (as for the decode entry
  * point), any page size >= 1, sm_scale > 0, q/k/v strides multiples of 8 and bases 16-byte
  * aligned, o strides multiples of 4 and base 8-byte aligned.
  * ---------------------------------------------------------------------------------------- */

@@ -137,6 +137,51 @@ def test_head_size_sweep(dev, seed):
     _close(o3.cpu(), oa.paged_decode(qd, kc, vc, table, kl))
 
 
+# head sizes above 128 (up to 256: one kernel instance, one wavefront per SIMD), e.g. the 192 / 128
+# of a multi-head-latent prefill and the 256 of some dense models; all three paths
+@pytest.mark.parametrize("d,dv", [(256, 256), (192, 128), (136, 136), (160, 256), (248, 8), (64, 192),
+                                  (256, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_large_head_sizes(dev, d, dv, dtype):
+    from dlcompiler_amd.kernels.paged_attention import paged_attention_fwd
+    from dlcompiler_amd.kernels.prefill_attention import context_attention_fwd
+
+    seed = d * 3 + dv
+    rng = random.Random(seed)
+    hkv = rng.choice([1, 2])
+    hq = hkv * rng.choice([1, 4])
+    gen = torch.Generator().manual_seed(seed)
+    lens = [rng.choice([1, 63, 64, 65, 130, 257]) for _ in range(3)]
+    nseq, T = len(lens), sum(lens)
+    start = torch.tensor([sum(lens[:i]) for i in range(nseq)], dtype=torch.int32)
+    sl = torch.tensor(lens, dtype=torch.int32)
+    q = torch.randn((T, hq, d), generator=gen).to(dtype)
+    k = torch.randn((T, hkv, d), generator=gen).to(dtype)
+    v = torch.randn((T, hkv, d), generator=gen).to(dtype)
+    o = torch.zeros_like(q, device=dev)
+    context_attention_fwd(q.to(dev), k.to(dev), v.to(dev), o, start.to(dev), sl.to(dev), max(lens))
+    _close(o.cpu(), oa.prefill_attention(q, k, v, start, sl))
+
+    for page in (16, 64, 48):
+        hist = [rng.choice([0, 17, 100, 300]) for _ in range(nseq)]
+        full = [a + b for a, b in zip(lens, hist)]
+        ks = [torch.randn((n, hkv, d), generator=gen).to(dtype) for n in full]
+        vs = [torch.randn((n, hkv, dv), generator=gen).to(dtype) for n in full]
+        kc, vc, table = oa.make_paged_cache(ks, vs, page, seed=seed, dtype=dtype)
+        ql, kl = torch.tensor(lens), torch.tensor(full)
+        o2 = torch.zeros((T, hq, dv), dtype=dtype, device=dev)
+        paged_attention_fwd(q.to(dev), kc.to(dev), vc.to(dev), o2, table.to(dev), start.to(dev),
+                            ql.to(dev), kl.to(dev), max(lens))
+        _close(o2.cpu(), oa.paged_prefill(q, kc, vc, table, start.long(), ql, kl))
+        qd = torch.randn((nseq, hq, d), generator=gen).to(dtype)
+        o3 = torch.zeros((nseq, hq, dv), dtype=dtype, device=dev)
+        window = rng.choice([None, 50])
+        paged_attention_fwd(qd.to(dev), kc.to(dev), vc.to(dev), o3, table.to(dev),
+                            torch.arange(nseq, device=dev), torch.ones(nseq, dtype=torch.int64, device=dev),
+                            kl.to(dev), 1, window_size=window)
+        _close(o3.cpu(), oa.paged_decode(qd, kc, vc, table, kl, window=window))
+
+
 def test_config_size_attention_repeats_bit_identically(dev):
     """Config-size prefill and paged decode, repeated: both kernels copy K/V into LDS with
     hand-issued loads and explicit waits; a missing wait would show as run-to-run differences."""

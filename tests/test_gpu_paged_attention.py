@@ -150,7 +150,7 @@ def test_unsupported_requests_raise(dev):
     with pytest.raises(NotImplementedError):
         paged_attention_fwd(*args(44))                       # head size not a multiple of 8
     with pytest.raises(NotImplementedError):
-        paged_attention_fwd(*args(136))                      # head size above 128
+        paged_attention_fwd(*args(264))                      # head size above 256
     q = torch.zeros((2, 4, 64), dtype=torch.float16, device=dev)
     kc = torch.zeros((4, 8, 2, 64), dtype=torch.float16, device=dev)
     with pytest.raises(NotImplementedError):                 # decode pages are multiples of 16
