@@ -244,9 +244,9 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // placement kernel reduces, else 128 (two passes)
 constexpr int kRouteMaxChunks = 256;
 inline int route_chunk_tokens(int64_t T) { return (T + 63) / 64 <= kRouteMaxChunks ? 64 : 128; }
-int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
-                              int K, int64_t ld_logits, int renormalize, int chunk_tokens,
-                              int32_t* chunk_counts, hipStream_t s);
+int launch_topk_softmax_count(const void* logits, int logits_dtype, float* weights, int32_t* ids,
+                              int64_t T, int E, int K, int64_t ld_logits, int renormalize,
+                              int chunk_tokens, int32_t* chunk_counts, hipStream_t s);
 
 // compute units of the device that is current on this thread (256 if it cannot be read), kept
 // per device: a process may drive GPUs of different sizes.  The table is filled lazily; two

@@ -550,9 +550,10 @@ extern "C" size_t dlb_moe_topk_softmax_align_ws_bytes(int64_t T, int E) {
   return (size_t)chunks * (size_t)E * sizeof(int32_t);
 }
 
-extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t* ids,
+extern "C" int dlb_moe_topk_softmax_align_f32(const void* logits, float* weights, int32_t* ids,
                                               int64_t T, int E, int K, int64_t ld_logits,
-                                              int renormalize, int block, int32_t* sorted_ids,
+                                              int logits_dtype, int renormalize, int block,
+                                              int32_t* sorted_ids,
                                               int64_t sorted_cap, int32_t* expert_ids,
                                               int64_t expert_ids_cap, int32_t* counts,
                                               int32_t* num_post_pad, void* ws, size_t ws_bytes,
@@ -560,6 +561,8 @@ extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weight
   using namespace dlb;
   if (T < 0 || E < 1 || K < 1 || K > E || ld_logits < E || block < 1) return DLB_ERR_BAD_ARG;
   if (K > 16 || E > kMaxE) return DLB_ERR_UNSUPPORTED;
+  if (logits_dtype != DLB_DTYPE_F32 && logits_dtype != DLB_DTYPE_BF16 && logits_dtype != DLB_DTYPE_F16)
+    return DLB_ERR_UNSUPPORTED;
   const int64_t numel = T * K;
   if (numel + (int64_t)E * block >= (int64_t)0x7fffffff) return DLB_ERR_UNSUPPORTED;
   const int chunk_tokens = route_chunk_tokens(T);
@@ -574,8 +577,8 @@ extern "C" int dlb_moe_topk_softmax_align_f32(const float* logits, float* weight
   hipStream_t s = (hipStream_t)stream;
   int32_t* chunk_counts = (int32_t*)ws;
   if (T > 0) {
-    const int st = launch_topk_softmax_count(logits, weights, ids, T, E, K, ld_logits, renormalize,
-                                             chunk_tokens, chunk_counts, s);
+    const int st = launch_topk_softmax_count(logits, logits_dtype, weights, ids, T, E, K, ld_logits,
+                                             renormalize, chunk_tokens, chunk_counts, s);
     if (st != DLB_OK) return st;
   } else {
     // no tokens: the single chunk is empty, but its row of the table is still read

@@ -36,29 +36,61 @@ __device__ __forceinline__ void row_step_max(uint32_t& key, uint32_t& tag) {
 }
 
 // The logits of one token, VPL consecutive experts per lane of its DPP row (-inf past E and for
-// dead rows).
-template <int VPL>
-__device__ __forceinline__ void load_token_logits(const float* __restrict__ logits, int64_t token,
+// dead rows).  LT = element type of the logits (fp32, or bf16 / fp16 converted on the way in: the
+// reference's fused gate kernel takes 16-bit logits and computes in fp32,
+// python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:44-46).
+template <int VPL, int LT>
+__device__ __forceinline__ void load_token_logits(const void* __restrict__ logits_v, int64_t token,
                                                   bool live, int E, int64_t ld, int vec_ok,
                                                   float (&v)[VPL]) {
   const int lane16 = threadIdx.x & 15;
   // every lane of a row takes the same branch; DPP rows never straddle tokens
   const float NEG_INF = -__builtin_inff();
   const int e0 = lane16 * VPL;
-  if (live && vec_ok) {
-    const f32x4* p = reinterpret_cast<const f32x4*>(logits + token * ld + e0);
+  if constexpr (LT == DLB_DTYPE_F32) {
+    const float* logits = (const float*)logits_v;
+    if (live && vec_ok) {
+      const f32x4* p = reinterpret_cast<const f32x4*>(logits + token * ld + e0);
 #pragma unroll
-    for (int q = 0; q < VPL / 4; ++q) {
-      const f32x4 t = p[q];
-      v[4 * q + 0] = t[0];
-      v[4 * q + 1] = t[1];
-      v[4 * q + 2] = t[2];
-      v[4 * q + 3] = t[3];
+      for (int q = 0; q < VPL / 4; ++q) {
+        const f32x4 t = p[q];
+        v[4 * q + 0] = t[0];
+        v[4 * q + 1] = t[1];
+        v[4 * q + 2] = t[2];
+        v[4 * q + 3] = t[3];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j)
+        v[j] = (live && e0 + j < E) ? logits[token * ld + e0 + j] : NEG_INF;
     }
   } else {
+    const unsigned short* logits = (const unsigned short*)logits_v;
+    if (live && vec_ok) {
+      const unsigned short* p = logits + token * ld + e0;
+      unsigned int w[VPL / 2];
+      if constexpr (VPL == 4) {
+        const u32x2 t = *reinterpret_cast<const u32x2*>(p);
+        w[0] = t[0];
+        w[1] = t[1];
+      } else {
 #pragma unroll
-    for (int j = 0; j < VPL; ++j)
-      v[j] = (live && e0 + j < E) ? logits[token * ld + e0 + j] : NEG_INF;
+        for (int q = 0; q < VPL / 8; ++q) {
+          const u32x4 t = reinterpret_cast<const u32x4*>(p)[q];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w[4 * q + i] = t[i];
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < VPL / 2; ++q) {
+        v[2 * q] = Elem<LT>::lo(w[q]);
+        v[2 * q + 1] = Elem<LT>::hi(w[q]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VPL; ++j)
+        v[j] = (live && e0 + j < E) ? Elem<LT>::load1(logits, token * ld + e0 + j) : NEG_INF;
+    }
   }
 }
 
@@ -154,14 +186,14 @@ __device__ __forceinline__ int32_t route_token(const float (&v)[VPL], float* __r
   return -1;
 }
 
-template <int VPL>
+template <int VPL, int LT>
 __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
-    const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
+    const void* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
     int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok, float* __restrict__ probs,
     int64_t* __restrict__ masks) {
   const int64_t token = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   float v[VPL];
-  load_token_logits<VPL>(logits, token, token < T, E, ld, vec_ok, v);
+  load_token_logits<VPL, LT>(logits, token, token < T, E, ld, vec_ok, v);
   route_token<VPL>(v, weights, ids, token, token < T, E, K, renorm, probs, masks, T);
 }
 
@@ -170,9 +202,9 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(
 // in LDS, then writes one row of the alignment's [chunks, E] count table -- the row of the
 // chunk made of exactly those tokens' K * 64 * PASSES flat routing slots.  Integer LDS adds
 // only, so the row does not depend on the order of execution.
-template <int VPL, int PASSES>
+template <int VPL, int PASSES, int LT>
 __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
-    const float* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
+    const void* __restrict__ logits, float* __restrict__ weights, int32_t* __restrict__ ids,
     int64_t T, int E, int K, int64_t ld, int renorm, int vec_ok,
     int32_t* __restrict__ chunk_counts) {
   __shared__ int32_t hist[256];
@@ -183,7 +215,7 @@ __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {  // all loads first: one memory round trip
     const int64_t token = first + pass * 64 + (threadIdx.x >> 4);
-    load_token_logits<VPL>(logits, token, token < T, E, ld, vec_ok, v[pass]);
+    load_token_logits<VPL, LT>(logits, token, token < T, E, ld, vec_ok, v[pass]);
   }
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
@@ -195,56 +227,78 @@ __global__ __launch_bounds__(1024) void moe_topk_softmax_count_kernel(
   for (int e = threadIdx.x; e < E; e += 1024) chunk_counts[(int64_t)blockIdx.x * E + e] = hist[e];
 }
 
+// whole-row vector loads of the logits: 16-byte aligned base, rows a whole number of 16-byte pieces
+bool logits_vector_ok(const void* logits, int dtype, int64_t ld) {
+  return aligned16(logits) && ld % (dtype == DLB_DTYPE_F32 ? 4 : 8) == 0;
+}
+
 }  // namespace
 
 // launch of the fused router + chunk histogram (used by the fused entry point of the alignment);
 // chunk_tokens is 64 or 128
-int launch_topk_softmax_count(const float* logits, float* weights, int32_t* ids, int64_t T, int E,
-                              int K, int64_t ld_logits, int renormalize, int chunk_tokens,
-                              int32_t* chunk_counts, hipStream_t s) {
+int launch_topk_softmax_count(const void* logits, int logits_dtype, float* weights, int32_t* ids,
+                              int64_t T, int E, int K, int64_t ld_logits, int renormalize,
+                              int chunk_tokens, int32_t* chunk_counts, hipStream_t s) {
   if (chunk_tokens != 64 && chunk_tokens != 128) return DLB_ERR_BAD_ARG;
   const dim3 grid((uint32_t)ceil_div(T, chunk_tokens)), block(1024);
-  const bool a16 = aligned16(logits) && (ld_logits % 4 == 0);
-#define DLB_LAUNCH_ROUTE_COUNT(VPL_, EFULL_)                                                     \
-  do {                                                                                           \
-    if (chunk_tokens == 64)                                                                      \
-      hipLaunchKernelGGL((moe_topk_softmax_count_kernel<VPL_, 1>), grid, block, 0, s, logits,    \
+  const bool a16 = logits_vector_ok(logits, logits_dtype, ld_logits);
+#define DLB_LAUNCH_ROUTE_COUNT_LT(VPL_, EFULL_, LT_)                                               \
+  do {                                                                                             \
+    if (chunk_tokens == 64)                                                                        \
+      hipLaunchKernelGGL((moe_topk_softmax_count_kernel<VPL_, 1, LT_>), grid, block, 0, s, logits, \
                          weights, ids, T, E, K, ld_logits, renormalize, (int)(a16 && E == EFULL_), \
-                         chunk_counts);                                                          \
-    else                                                                                         \
-      hipLaunchKernelGGL((moe_topk_softmax_count_kernel<VPL_, 2>), grid, block, 0, s, logits,    \
+                         chunk_counts);                                                            \
+    else                                                                                           \
+      hipLaunchKernelGGL((moe_topk_softmax_count_kernel<VPL_, 2, LT_>), grid, block, 0, s, logits, \
                          weights, ids, T, E, K, ld_logits, renormalize, (int)(a16 && E == EFULL_), \
-                         chunk_counts);                                                          \
+                         chunk_counts);                                                            \
+  } while (0)
+#define DLB_LAUNCH_ROUTE_COUNT(VPL_, EFULL_)                                          \
+  do {                                                                                \
+    if (logits_dtype == DLB_DTYPE_F32) DLB_LAUNCH_ROUTE_COUNT_LT(VPL_, EFULL_, DLB_DTYPE_F32);      \
+    else if (logits_dtype == DLB_DTYPE_BF16) DLB_LAUNCH_ROUTE_COUNT_LT(VPL_, EFULL_, DLB_DTYPE_BF16); \
+    else DLB_LAUNCH_ROUTE_COUNT_LT(VPL_, EFULL_, DLB_DTYPE_F16);                                    \
   } while (0)
   if (E <= 64) DLB_LAUNCH_ROUTE_COUNT(4, 64);
   else if (E <= 128) DLB_LAUNCH_ROUTE_COUNT(8, 128);
   else DLB_LAUNCH_ROUTE_COUNT(16, 256);
 #undef DLB_LAUNCH_ROUTE_COUNT
+#undef DLB_LAUNCH_ROUTE_COUNT_LT
   return launch_status();
 }
 
 }  // namespace dlb
 
-extern "C" int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids,
+extern "C" int dlb_moe_topk_softmax_f32(const void* logits, float* weights, int32_t* ids,
                                         float* probs, int64_t* masks, int64_t T, int E, int K,
-                                        int64_t ld_logits, int renormalize, void* stream) {
+                                        int64_t ld_logits, int logits_dtype, int renormalize,
+                                        void* stream) {
   using namespace dlb;
   if (T < 0 || E < 1 || K < 1 || K > E || ld_logits < E) return DLB_ERR_BAD_ARG;
   if (K > 16 || E > 256) return DLB_ERR_UNSUPPORTED;
+  if (logits_dtype != DLB_DTYPE_F32 && logits_dtype != DLB_DTYPE_BF16 && logits_dtype != DLB_DTYPE_F16)
+    return DLB_ERR_UNSUPPORTED;
   if (T == 0) return DLB_OK;
   if (!logits || !weights || !ids) return DLB_ERR_BAD_ARG;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)ceil_div(T, 16)), block(256);
-  const bool a16 = aligned16(logits) && (ld_logits % 4 == 0);
-  if (E <= 64) {
-    hipLaunchKernelGGL(moe_topk_softmax_kernel<4>, grid, block, 0, s, logits, weights, ids, T, E,
-                       K, ld_logits, renormalize, (int)(a16 && E == 64), probs, masks);
-  } else if (E <= 128) {
-    hipLaunchKernelGGL(moe_topk_softmax_kernel<8>, grid, block, 0, s, logits, weights, ids, T, E,
-                       K, ld_logits, renormalize, (int)(a16 && E == 128), probs, masks);
-  } else {
-    hipLaunchKernelGGL(moe_topk_softmax_kernel<16>, grid, block, 0, s, logits, weights, ids, T, E,
-                       K, ld_logits, renormalize, (int)(a16 && E == 256), probs, masks);
-  }
+  const bool a16 = logits_vector_ok(logits, logits_dtype, ld_logits);
+#define DLB_LAUNCH_ROUTE(LT_)                                                                      \
+  do {                                                                                             \
+    if (E <= 64)                                                                                   \
+      hipLaunchKernelGGL((moe_topk_softmax_kernel<4, LT_>), grid, block, 0, s, logits, weights, ids, \
+                         T, E, K, ld_logits, renormalize, (int)(a16 && E == 64), probs, masks);    \
+    else if (E <= 128)                                                                             \
+      hipLaunchKernelGGL((moe_topk_softmax_kernel<8, LT_>), grid, block, 0, s, logits, weights, ids, \
+                         T, E, K, ld_logits, renormalize, (int)(a16 && E == 128), probs, masks);   \
+    else                                                                                           \
+      hipLaunchKernelGGL((moe_topk_softmax_kernel<16, LT_>), grid, block, 0, s, logits, weights,   \
+                         ids, T, E, K, ld_logits, renormalize, (int)(a16 && E == 256), probs,      \
+                         masks);                                                                   \
+  } while (0)
+  if (logits_dtype == DLB_DTYPE_F32) DLB_LAUNCH_ROUTE(DLB_DTYPE_F32);
+  else if (logits_dtype == DLB_DTYPE_BF16) DLB_LAUNCH_ROUTE(DLB_DTYPE_BF16);
+  else DLB_LAUNCH_ROUTE(DLB_DTYPE_F16);
+#undef DLB_LAUNCH_ROUTE
   return launch_status();
 }

@@ -12,6 +12,17 @@ import torch
 from .. import _lib
 
 
+def _router_logits(logits: torch.Tensor) -> torch.Tensor:
+    """fp32, bf16 and fp16 logits are read as they are (the kernels convert on the way in, as the
+    reference's gate kernel does, python/dlBLAS/dlblas/kernels/topk_gating_fwd_part1.py:44-46);
+    anything else is converted to fp32 first."""
+    if logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        logits = logits.float()
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    return logits
+
+
 def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True,
                      return_probs: bool = False, return_masks: bool = False):
     """softmax(logits, fp32) -> top-k -> (optionally) weights / weights.sum(-1).
@@ -27,10 +38,7 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True,
     T, E = logits.shape
     if not 1 <= k <= E:
         raise ValueError(f"need 1 <= k <= num_experts, got k={k}, E={E}")
-    if logits.dtype != torch.float32:
-        logits = logits.float()
-    if logits.stride(1) != 1:
-        logits = logits.contiguous()
+    logits = _router_logits(logits)
     weights = torch.empty((T, k), dtype=torch.float32, device=logits.device)
     ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
     probs = torch.empty((T, E), dtype=torch.float32, device=logits.device) if return_probs else None
@@ -43,7 +51,7 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True,
                                               probs.data_ptr() if return_probs else None,
                                               masks.data_ptr() if return_masks else None, T, E, k,
                                               logits.stride(0) if T > 1 else E,
-                                              int(bool(renormalize)),
+                                              _lib.torch_dtype_code(logits.dtype), int(bool(renormalize)),
                                               _lib.current_stream_ptr(logits.device))
         _lib.check(st, "dlb_moe_topk_softmax_f32")
     out = (weights, ids)
@@ -126,10 +134,7 @@ def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_ex
         weights, ids = moe_topk_softmax(logits, k, renormalize)
         return (weights, ids) + tuple(moe_align_block_size(ids, block_size, num_experts,
                                                            return_counts=return_counts))
-    if logits.dtype != torch.float32:
-        logits = logits.float()
-    if logits.stride(1) != 1:
-        logits = logits.contiguous()
+    logits = _router_logits(logits)
     dev = logits.device
     numel = T * k
     cap = numel + E * (block_size - 1)
@@ -156,7 +161,8 @@ def moe_topk_softmax_align(logits: torch.Tensor, k: int, block_size: int, num_ex
     with _lib.device_guard(dev):
         st = lib.dlb_moe_topk_softmax_align_f32(
             logits.data_ptr(), weights.data_ptr(), ids.data_ptr(), T, E, k,
-            logits.stride(0) if T > 1 else E, int(bool(renormalize)), block_size,
+            logits.stride(0) if T > 1 else E, _lib.torch_dtype_code(logits.dtype), int(bool(renormalize)),
+            block_size,
             sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk, counts.data_ptr(),
             num_post.data_ptr(),
             ws.data_ptr(), ws.numel() * 4, _lib.current_stream_ptr(dev))

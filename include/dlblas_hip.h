@@ -37,7 +37,7 @@ extern "C" {
 
 /* ABI version: bumped whenever a signature below changes; dlb_version() returns the value the
  * library was built with, and a binding should refuse a library whose version differs. */
-#define DLB_ABI_VERSION 3
+#define DLB_ABI_VERSION 4
 int dlb_version(void);
 
 /* Index arrays (block tables, sequence lengths, start offsets) are read in the integer width the
@@ -64,7 +64,9 @@ int dlb_silu_and_mul(const void* x, void* out, int64_t M, int64_t N, int64_t ld_
  * (tests/kernels/test_fused_moe.py:213-216: softmax(fp32) then torch.topk; renormalise
  * kernels/fused_moe.py:322-323) and the fused softmax+argmax of
  * kernels/topk_gating_fwd_part1.py:24-60.
- *   logits  fp32 [T, E], row stride ld_logits
+ *   logits  [T, E] of type logits_dtype (DLB_DTYPE_F32, or BF16 / F16 converted to fp32 on the
+ *           way in, as the reference's gate kernel does, topk_gating_fwd_part1.py:44-46),
+ *           row stride ld_logits (elements)
  *   weights fp32 [T, K] (contiguous) ; ids int32 [T, K] (contiguous)
  * Selection is on the logits, descending, ties to the LOWEST expert index; weights are
  * p = exp(l - max) / sum(exp(l - max)) of the selected experts, divided by their sum when
@@ -75,9 +77,9 @@ int dlb_silu_and_mul(const void* x, void* out, int64_t M, int64_t N, int64_t ld_
  *   masks int64 [K, T, E] (contiguous): masks[r, t, :] is the one-hot row of the r-th selected
  *         expert of token t (the reference's K rounds of argmax / overwrite, :52-60).
  * ---------------------------------------------------------------------------------------- */
-int dlb_moe_topk_softmax_f32(const float* logits, float* weights, int32_t* ids, float* probs,
+int dlb_moe_topk_softmax_f32(const void* logits, float* weights, int32_t* ids, float* probs,
                              int64_t* masks, int64_t T, int E, int K, int64_t ld_logits,
-                             int renormalize, void* stream);
+                             int logits_dtype, int renormalize, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * moe_align_block_size: per-expert counts, expert-sorted flat slot ids padded per expert to a
@@ -146,8 +148,9 @@ int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int 
  * 32768 tokens: make the two calls then.
  * ---------------------------------------------------------------------------------------- */
 size_t dlb_moe_topk_softmax_align_ws_bytes(int64_t T, int E);
-int dlb_moe_topk_softmax_align_f32(const float* logits, float* weights, int32_t* ids, int64_t T,
-                                   int E, int K, int64_t ld_logits, int renormalize, int block,
+int dlb_moe_topk_softmax_align_f32(const void* logits, float* weights, int32_t* ids, int64_t T,
+                                   int E, int K, int64_t ld_logits, int logits_dtype,
+                                   int renormalize, int block,
                                    int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids,
                                    int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
                                    void* ws, size_t ws_bytes, void* stream);

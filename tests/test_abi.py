@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_status_strings():
     lib = _lib.load()
-    assert lib.dlb_version() == _lib.ABI_VERSION == 3
+    assert lib.dlb_version() == _lib.ABI_VERSION == 4
     assert lib.dlb_status_string(0) == b"ok"
     for code in (-1, -2, -3, -4, -99):
         assert lib.dlb_status_string(code)
@@ -57,8 +57,9 @@ def test_argument_validation_needs_no_gpu():
     assert lib.dlb_silu_and_mul(None, None, -1, 8, 16, 8, 0, None) == -1
     assert lib.dlb_silu_and_mul(None, None, 4, 8, 8, 8, 0, None) == -1  # ld_x < 2N
     assert lib.dlb_silu_and_mul(None, None, 0, 8, 16, 8, 0, None) == 0  # empty is fine
-    assert lib.dlb_moe_topk_softmax_f32(None, None, None, None, None, 4, 64, 65, 64, 1, None) == -1
-    assert lib.dlb_moe_topk_softmax_f32(None, None, None, None, None, 4, 512, 2, 512, 1, None) == -2
+    assert lib.dlb_moe_topk_softmax_f32(None, None, None, None, None, 4, 64, 65, 64, 2, 1, None) == -1
+    assert lib.dlb_moe_topk_softmax_f32(None, None, None, None, None, 4, 512, 2, 512, 2, 1, None) == -2
+    assert lib.dlb_moe_topk_softmax_f32(None, None, None, None, None, 4, 64, 2, 64, 7, 1, None) == -2  # logits type
     assert lib.dlb_moe_align_ws_bytes(98304, 64) > 0
 
 

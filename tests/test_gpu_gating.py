@@ -182,3 +182,28 @@ def test_fused_router_and_alignment_equals_the_two_calls(dev, T, E, k, block, re
         os_, oe, otot, _ = og.align_block_size(oids, block, E)
         assert torch.equal(sorted_ids.cpu(), os_) and torch.equal(expert_ids.cpu(), oe)
         assert int(npad.item()) == int(otot.item())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k", [(1000, 64, 6), (333, 128, 8), (77, 256, 4), (50, 60, 3), (40, 100, 2)])
+def test_sixteen_bit_logits_are_read_as_they_are(dev, dtype, T, E, k):
+    """bf16 / fp16 router logits go to the kernels unconverted (the reference's gate kernel takes
+    them too, topk_gating_fwd_part1.py:44-46): same results, bit for bit, as the fp32 copy."""
+    from dlcompiler_amd.kernels.moe_gating import moe_topk_softmax, moe_topk_softmax_align
+
+    g = torch.Generator().manual_seed(T + E)
+    wide = torch.randn((T, E + 8), generator=g).to(dtype).to(dev)
+    for logits in (wide[:, :E].contiguous(), wide[:, :E]):       # vector rows, and a strided view
+        ref = moe_topk_softmax(logits.float(), k, True, return_probs=True)
+        got = moe_topk_softmax(logits, k, True, return_probs=True)
+        for a, b in zip(ref, got):
+            assert torch.equal(a, b)
+        ref = moe_topk_softmax_align(logits.float(), k, 64, return_counts=True)
+        got = moe_topk_softmax_align(logits, k, 64, return_counts=True)
+        for a, b in zip(ref, got):
+            assert torch.equal(a, b)
+    # and against the oracle on the same 16-bit values
+    rw, rids = og.topk_softmax(wide[:, :E].cpu(), k)
+    w, ids = moe_topk_softmax(wide[:, :E], k)
+    assert torch.equal(ids.cpu(), rids)
+    torch.testing.assert_close(w.cpu(), rw, rtol=1e-6, atol=0)
