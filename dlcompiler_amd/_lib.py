@@ -14,7 +14,7 @@ _PKG_DIR = Path(__file__).resolve().parent
 DEFAULT_LIB_PATH = _PKG_DIR / "lib" / "libdlblas_hip.so"
 
 DLB_OK = 0
-ABI_VERSION = 4  # DLB_ABI_VERSION of include/dlblas_hip.h this binding was written against
+ABI_VERSION = 5  # DLB_ABI_VERSION of include/dlblas_hip.h this binding was written against
 DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 
 # name -> (restype, argtypes); must list every symbol include/dlblas_hip.h declares
@@ -26,15 +26,15 @@ SIGNATURES = {
     "dlb_moe_topk_softmax_f32": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int64, c_int, c_int,
                                                           c_void_p]),
     "dlb_moe_align_ws_bytes": (c_size_t, [c_int64, c_int]),
-    "dlb_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+    "dlb_moe_align_block_size": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int64,
                                          c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                          c_size_t, c_void_p]),
-    "dlb_moe_align_quant_fp8": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+    "dlb_moe_align_quant_fp8": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int64,
                                         c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_size_t,
                                         c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int64,
                                         c_int64, c_int64, c_int, c_void_p]),
     "dlb_moe_align_block_size_static_max_numel": (c_int64, []),
-    "dlb_moe_align_block_size_static": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_int64,
+    "dlb_moe_align_block_size_static": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_void_p, c_int64,
                                                 c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "dlb_moe_topk_softmax_align_ws_bytes": (c_size_t, [c_int64, c_int]),
     "dlb_moe_topk_softmax_align_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int,

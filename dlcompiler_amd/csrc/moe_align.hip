@@ -47,7 +47,7 @@ __host__ __device__ inline int64_t num_chunks(int64_t numel) {
   return numel > 0 ? (numel + c - 1) / c : 1;
 }
 
-__global__ __launch_bounds__(kThreads) void align_count_kernel(const int32_t* __restrict__ ids,
+__global__ __launch_bounds__(kThreads) void align_count_kernel(const IdxArray ids,
                                                                int64_t numel, int E, int chunk_ids,
                                                                int32_t* __restrict__ chunk_counts) {
   __shared__ int32_t hist[kMaxE];
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
 }
 
 __global__ __launch_bounds__(kThreads) void align_place_kernel(
-    const int32_t* __restrict__ ids, int64_t numel, int E,
+    const IdxArray ids, int64_t numel, int E,
     const int32_t* __restrict__ chunk_start, int32_t* __restrict__ sorted_ids) {
   __shared__ int32_t cursor[kMaxE];           // next free slot per expert for this chunk
   __shared__ int32_t wave_cnt[kWaves][kMaxE];  // per-tile, per-wave counts
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void align_place_kernel(
 // one extra workgroup emits what the scan kernel emits (counts, block -> expert ids, pad slots,
 // tails, padded total).  The table is only read here.
 struct PlaceParams {
-  const int32_t* ids;
+  IdxArray ids;  // int32 or int64 (the routing ids as torch.topk returns them)
   int64_t numel;
   int E, block;
   const int32_t* chunk_counts;
@@ -216,7 +216,7 @@ struct PlaceParams {
 
 // the work of workgroup `me` (0 .. chunks) of the fused scan + placement
 __device__ __forceinline__ void align_place_fused_block(const PlaceParams& pp, const int me) {
-  const int32_t* __restrict__ ids = pp.ids;
+  const IdxArray ids = pp.ids;
   const int64_t numel = pp.numel;
   const int E = pp.E, block = pp.block, chunks = pp.chunks, chunk_ids = pp.chunk_ids;
   const int32_t* __restrict__ chunk_counts = pp.chunk_counts;
@@ -396,7 +396,7 @@ namespace dlb {
 namespace {
 
 // argument checks shared by the two alignment entry points (everything but the scratch)
-int check_align_args(const int32_t* topk_ids, int64_t numel, int E, int block,
+int check_align_args(const void* topk_ids, int64_t numel, int E, int block,
                      const int32_t* sorted_ids, int64_t sorted_cap, const int32_t* expert_ids,
                      int64_t expert_ids_cap, const int32_t* num_post_pad) {
   if (numel < 0 || E < 1 || block < 1) return DLB_ERR_BAD_ARG;
@@ -411,7 +411,7 @@ int check_align_args(const int32_t* topk_ids, int64_t numel, int E, int block,
 
 // the launches of the alignment; chunk_counts holds num_chunks(numel) x E int32, every word of
 // which the counting pass overwrites before anything reads it (nothing has to start at zero)
-int launch_align(const int32_t* topk_ids, int64_t numel, int E, int block, int32_t* sorted_ids,
+int launch_align(const IdxArray topk_ids, int64_t numel, int E, int block, int32_t* sorted_ids,
                  int64_t sorted_cap, int32_t* expert_ids, int64_t expert_ids_cap, int32_t* counts,
                  int32_t* num_post_pad, int32_t* chunk_counts, hipStream_t s,
                  const QuantParams* quant = nullptr, int quant_dtype = DLB_DTYPE_BF16) {
@@ -477,7 +477,7 @@ int static_scratch(int32_t** out) {
 }  // namespace
 }  // namespace dlb
 
-extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int block,
+extern "C" int dlb_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t numel, int E, int block,
                                         int32_t* sorted_ids, int64_t sorted_cap,
                                         int32_t* expert_ids, int64_t expert_ids_cap,
                                         int32_t* counts, int32_t* num_post_pad, void* ws,
@@ -487,11 +487,12 @@ extern "C" int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, 
                                   expert_ids_cap, num_post_pad);
   if (st != DLB_OK) return st;
   if (!ws || ws_bytes < dlb_moe_align_ws_bytes(numel, E)) return DLB_ERR_WORKSPACE;
-  return launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
-                      expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream);
+  return launch_align(idx_array(topk_ids, ids_int64 ? 1 : 0, 0), numel, E, block, sorted_ids, sorted_cap,
+                      expert_ids, expert_ids_cap, counts, num_post_pad, (int32_t*)ws,
+                      (hipStream_t)stream);
 }
 
-extern "C" int dlb_moe_align_quant_fp8(const int32_t* topk_ids, int64_t numel, int E, int block,
+extern "C" int dlb_moe_align_quant_fp8(const void* topk_ids, int ids_int64, int64_t numel, int E, int block,
                                        int32_t* sorted_ids, int64_t sorted_cap,
                                        int32_t* expert_ids, int64_t expert_ids_cap,
                                        int32_t* counts, int32_t* num_post_pad, void* ws,
@@ -506,12 +507,13 @@ extern "C" int dlb_moe_align_quant_fp8(const int32_t* topk_ids, int64_t numel, i
   QuantParams q;
   const int sq = fill_quant_params(q, x, xq, xs, M, K, ld_x, ld_q, ld_s, dtype);
   if (sq != DLB_OK) return sq;
+  const IdxArray ids = idx_array(topk_ids, ids_int64 ? 1 : 0, 0);
   if (num_chunks(numel) <= kFusedChunks)
-    return launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+    return launch_align(ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
                         expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream, &q,
                         dtype);
   // more routing slots than the fused placement takes: the separate launches
-  const int sa = launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
+  const int sa = launch_align(ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
                               expert_ids_cap, counts, num_post_pad, (int32_t*)ws, (hipStream_t)stream);
   if (sa != DLB_OK) return sa;
   return dlb_per_token_group_quant_fp8(x, xq, xs, M, K, ld_x, ld_q, ld_s, dtype, stream);
@@ -521,8 +523,8 @@ extern "C" int64_t dlb_moe_align_block_size_static_max_numel(void) {
   return (int64_t)dlb::kStaticChunks * dlb::kChunk;  // = kFusedChunks chunks of the largest size
 }
 
-extern "C" int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int E,
-                                               int block, int32_t* sorted_ids, int64_t sorted_cap,
+extern "C" int dlb_moe_align_block_size_static(const void* topk_ids, int ids_int64, int64_t numel,
+                                               int E, int block, int32_t* sorted_ids, int64_t sorted_cap,
                                                int32_t* expert_ids, int64_t expert_ids_cap,
                                                int32_t* counts, int32_t* num_post_pad,
                                                void* stream) {
@@ -535,8 +537,9 @@ extern "C" int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t 
   int32_t* chunk_counts = nullptr;
   const int sp = static_scratch(&chunk_counts);
   if (sp != DLB_OK) return sp;
-  return launch_align(topk_ids, numel, E, block, sorted_ids, sorted_cap, expert_ids,
-                      expert_ids_cap, counts, num_post_pad, chunk_counts, (hipStream_t)stream);
+  return launch_align(idx_array(topk_ids, ids_int64 ? 1 : 0, 0), numel, E, block, sorted_ids, sorted_cap,
+                      expert_ids, expert_ids_cap, counts, num_post_pad, chunk_counts,
+                      (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -582,10 +585,10 @@ extern "C" int dlb_moe_topk_softmax_align_f32(const void* logits, float* weights
     if (st != DLB_OK) return st;
   } else {
     // no tokens: the single chunk is empty, but its row of the table is still read
-    hipLaunchKernelGGL(align_count_kernel, dim3(1), dim3(kThreads), 0, s, ids, (int64_t)0, E, kChunk,
-                       chunk_counts);
+    hipLaunchKernelGGL(align_count_kernel, dim3(1), dim3(kThreads), 0, s, IdxArray{ids, 0}, (int64_t)0, E,
+                       kChunk, chunk_counts);
   }
-  const PlaceParams pp = {ids,        numel,      E,          block,          chunk_counts, (int)chunks,
+  const PlaceParams pp = {IdxArray{ids, 0}, numel, E, block, chunk_counts, (int)chunks,
                           chunk_tokens * K, sorted_ids, sorted_cap, expert_ids, expert_ids_cap,
                           counts,     num_post_pad};
   hipLaunchKernelGGL(align_place_fused_kernel, dim3((uint32_t)chunks + 1), dim3(kThreads), 0, s, pp);

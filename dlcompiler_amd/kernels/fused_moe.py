@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from .. import _lib
-from .moe_gating import moe_align_block_size
+from .moe_gating import moe_align_block_size, routing_ids
 
 # rows per grouped-GEMM workgroup tile = alignment block of the routing; tiles skip 32-row groups
 # that hold padding only, so the matrix work follows the routed rows in steps of 32
@@ -50,10 +50,7 @@ def _align_and_quant(topk_ids: torch.Tensor, block: int, num_experts: int, x: to
     """:func:`moe_align_block_size` (with counts) and :func:`per_token_group_quant_fp8` as one
     native call of two launches: the quantiser runs in the launch of the placement pass.
     Returns ``(sorted_token_ids, counts, xq, xs)``."""
-    ids = topk_ids.reshape(-1)
-    if ids.dtype != torch.int32:
-        ids = ids.to(torch.int32)
-    ids = ids.contiguous()
+    ids = routing_ids(topk_ids)
     if x.stride(1) != 1:
         x = x.contiguous()
     M, K = x.shape
@@ -75,7 +72,8 @@ def _align_and_quant(topk_ids: torch.Tensor, block: int, num_experts: int, x: to
     xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=dev)
     with _lib.device_guard(dev):
         st = lib.dlb_moe_align_quant_fp8(
-            ids.data_ptr(), numel, num_experts, block, sorted_ids.data_ptr(), cap,
+            ids.data_ptr(), int(ids.dtype == torch.int64), numel, num_experts, block,
+            sorted_ids.data_ptr(), cap,
             expert_ids.data_ptr(), nblk, counts.data_ptr(), num_post.data_ptr(), ws.data_ptr(),
             ws.numel() * 4, x.data_ptr(), xq.data_ptr(), xs.data_ptr(), M, K,
             x.stride(0) if M > 1 else K, K, K // 128, _lib.torch_dtype_code(x.dtype),

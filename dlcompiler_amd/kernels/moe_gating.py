@@ -62,6 +62,15 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True,
     return out
 
 
+def routing_ids(topk_ids: torch.Tensor) -> torch.Tensor:
+    """The flat routing ids as the alignment kernels read them: int32 and int64 (what
+    ``torch.topk`` returns) pass unconverted, any other integer type becomes int32."""
+    ids = topk_ids.reshape(-1)
+    if ids.dtype not in (torch.int32, torch.int64):
+        ids = ids.to(torch.int32)
+    return ids.contiguous()
+
+
 def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int,
                          return_counts: bool = False):
     """Group the flat routing slots ``i = token * k + j`` by expert, padded to ``block_size``.
@@ -79,10 +88,7 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     _lib.require_cuda(topk_ids)
     if block_size < 1 or num_experts < 1:
         raise ValueError("block_size and num_experts must be positive")
-    ids = topk_ids.reshape(-1)
-    if ids.dtype != torch.int32:
-        ids = ids.to(torch.int32)
-    ids = ids.contiguous()
+    ids = routing_ids(topk_ids)
     numel = ids.numel()
     dev = ids.device
     cap = numel + num_experts * (block_size - 1)
@@ -98,7 +104,8 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     buf = torch.empty((total,), dtype=torch.int32, device=dev)
     sorted_ids, expert_ids, num_post, counts, ws = (buf[o:o + n] for o, n in zip(offs, sizes))
     with _lib.device_guard(dev):
-        st = lib.dlb_moe_align_block_size(ids.data_ptr(), numel, num_experts, block_size,
+        st = lib.dlb_moe_align_block_size(ids.data_ptr(), int(ids.dtype == torch.int64), numel,
+                                          num_experts, block_size,
                                           sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), nblk,
                                           counts.data_ptr(), num_post.data_ptr(), ws.data_ptr(),
                                           ws.numel() * 4, _lib.current_stream_ptr(dev))

@@ -37,7 +37,7 @@ extern "C" {
 
 /* ABI version: bumped whenever a signature below changes; dlb_version() returns the value the
  * library was built with, and a binding should refuse a library whose version differs. */
-#define DLB_ABI_VERSION 4
+#define DLB_ABI_VERSION 5
 int dlb_version(void);
 
 /* Index arrays (block tables, sequence lengths, start offsets) are read in the integer width the
@@ -87,7 +87,9 @@ int dlb_moe_topk_softmax_f32(const void* logits, float* weights, int32_t* ids, f
  * Replaces the routing bookkeeping of fused_moe: argsort + get_start_end/_start_end_kernel,
  * kernels/fused_moe.py:238-293,314-320 (the pad-to-block layout itself has no reference
  * counterpart).
- *   topk_ids    int32 [numel]  (flat index i = token * K + j); ids outside [0, E) are dropped
+ *   topk_ids    int32 [numel], or int64 with ids_int64 != 0 (what torch.topk returns and the
+ *               reference's callers hand over, kernels/fused_moe.py:296-320); flat index
+ *               i = token * K + j; ids outside [0, E) are dropped
  *   sorted_ids  int32 [sorted_cap], sorted_cap >= numel + E * (block - 1):
  *               expert segments in expert order, each a multiple of `block` long, holding the
  *               flat indices of that expert ASCENDING, then pad slots; every slot that is not
@@ -100,7 +102,7 @@ int dlb_moe_topk_softmax_f32(const void* logits, float* weights, int32_t* ids, f
  * 1 <= E <= 256, block >= 1, numel < 2^31 - E * block.
  * ---------------------------------------------------------------------------------------- */
 size_t dlb_moe_align_ws_bytes(int64_t numel, int E);
-int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int block,
+int dlb_moe_align_block_size(const void* topk_ids, int ids_int64, int64_t numel, int E, int block,
                              int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids,
                              int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
                              void* ws, size_t ws_bytes, void* stream);
@@ -111,7 +113,7 @@ int dlb_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int E, int 
  * the two functions, bit for bit; it is what fused_moe_fp8 runs in front of its GEMMs (the
  * reference sorts inside fused_moe as well, kernels/fused_moe.py:314-320).  Inputs beyond 524288
  * routing slots fall back to the separate launches. */
-int dlb_moe_align_quant_fp8(const int32_t* topk_ids, int64_t numel, int E, int block,
+int dlb_moe_align_quant_fp8(const void* topk_ids, int ids_int64, int64_t numel, int E, int block,
                             int32_t* sorted_ids, int64_t sorted_cap, int32_t* expert_ids,
                             int64_t expert_ids_cap, int32_t* counts, int32_t* num_post_pad,
                             void* ws, size_t ws_bytes, const void* x, void* xq, float* xs,
@@ -132,7 +134,7 @@ int dlb_moe_align_quant_fp8(const int32_t* topk_ids, int64_t numel, int E, int b
  * every device outside stream capture before the entry point is used in a captured region.
  * ---------------------------------------------------------------------------------------- */
 int64_t dlb_moe_align_block_size_static_max_numel(void);
-int dlb_moe_align_block_size_static(const int32_t* topk_ids, int64_t numel, int E, int block,
+int dlb_moe_align_block_size_static(const void* topk_ids, int ids_int64, int64_t numel, int E, int block,
                                     int32_t* sorted_ids, int64_t sorted_cap,
                                     int32_t* expert_ids, int64_t expert_ids_cap, int32_t* counts,
                                     int32_t* num_post_pad, void* stream);

@@ -29,7 +29,7 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_status_strings():
     lib = _lib.load()
-    assert lib.dlb_version() == _lib.ABI_VERSION == 4
+    assert lib.dlb_version() == _lib.ABI_VERSION == 5
     assert lib.dlb_status_string(0) == b"ok"
     for code in (-1, -2, -3, -4, -99):
         assert lib.dlb_status_string(code)
@@ -99,9 +99,9 @@ def test_launcher_and_fused_prepare_argument_checks_need_no_gpu():
     assert launcher(mask=8) == -1                 # three index arrays: bits 0..2
     assert launcher(num_experts=300, local=300) == -2
     # alignment + quantisation in one call: the checks of both halves apply before any launch
-    assert lib.dlb_moe_align_quant_fp8(one, 64, 8, 128, one, 64 + 8 * 127, one, 9, one, one, None, 0,
+    assert lib.dlb_moe_align_quant_fp8(one, 0, 64, 8, 128, one, 64 + 8 * 127, one, 9, one, one, None, 0,
                                        one, one, one, 32, 256, 256, 256, 2, 0, None) == -4  # no workspace
-    assert lib.dlb_moe_align_quant_fp8(one, 64, 8, 128, one, 10, one, 9, one, one, one, 1 << 20,
+    assert lib.dlb_moe_align_quant_fp8(one, 0, 64, 8, 128, one, 10, one, 9, one, one, one, 1 << 20,
                                        one, one, one, 32, 256, 256, 256, 2, 0, None) == -1  # sorted_cap too small
-    assert lib.dlb_moe_align_quant_fp8(one, 64, 8, 128, one, 64 + 8 * 127, one, 9, one, one, one, 1 << 20,
+    assert lib.dlb_moe_align_quant_fp8(one, 0, 64, 8, 128, one, 64 + 8 * 127, one, 9, one, one, one, 1 << 20,
                                        one, one, one, 32, 200, 200, 200, 1, 0, None) == -2  # K % 128

@@ -245,3 +245,19 @@ def test_zero_tokens(dev):
                               torch.empty((0,), dtype=torch.int64, device=dev), none, none, None,
                               False, 2, 0, 0, True, True)
     torch.cuda.synchronize()
+
+
+def test_int64_topk_ids(dev):
+    """The ids of torch.topk (int64) go through fused_moe and fused_moe_fp8 unconverted."""
+    from dlcompiler_amd.kernels.fused_moe import fused_moe, fused_moe_fp8
+    from oracle import fp8 as ofp8
+
+    x, w1, w2, tw, ids = _inputs(200, 256, 128, 8, 2, 21, torch.bfloat16)
+    d = [t.to(dev) for t in (x, w1, w2, tw)]
+    a = fused_moe(*d, ids.to(dev), topk=2)
+    b = fused_moe(*d, ids.long().to(dev), topk=2)
+    assert torch.equal(a, b)
+    w1q, w1s = ofp8.block_quant_weight(w1.float())
+    w2q, w2s = ofp8.block_quant_weight(w2.float())
+    q = [t.to(dev) for t in (x, w1q, w1s, w2q, w2s, tw)]
+    assert torch.equal(fused_moe_fp8(*q, ids.to(dev), 2), fused_moe_fp8(*q, ids.long().to(dev), 2))

@@ -207,3 +207,20 @@ def test_sixteen_bit_logits_are_read_as_they_are(dev, dtype, T, E, k):
     w, ids = moe_topk_softmax(wide[:, :E], k)
     assert torch.equal(ids.cpu(), rids)
     torch.testing.assert_close(w.cpu(), rw, rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("T,E,k,block", [(4096, 64, 6, 128), (300, 8, 2, 16), (1, 4, 1, 64)])
+def test_int64_routing_ids_are_read_as_they_are(dev, T, E, k, block):
+    """torch.topk hands over int64 ids and the reference's fused_moe takes them
+    (fused_moe.py:296-320): the alignment reads either width, same results bit for bit; ids of
+    experts held elsewhere (out of range, negative) are dropped in both."""
+    from dlcompiler_amd.kernels.moe_gating import moe_align_block_size
+
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.randint(-1, E + 2, (T, k), generator=g)            # int64, some out of range
+    a = moe_align_block_size(ids.to(torch.int32).to(dev), block, E, return_counts=True)
+    b = moe_align_block_size(ids.to(dev), block, E, return_counts=True)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    rs, re_, rn, rc = og.align_block_size(ids, block, E)
+    assert torch.equal(b[3].cpu(), rc.to(torch.int32)) and int(b[2].item()) == int(rn.item())

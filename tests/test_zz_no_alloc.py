@@ -25,14 +25,14 @@ def _align_pair(ids, E, block):
     cap, nblk, s0, e0, c0, n0 = _buffers(numel, E, block, dev)
     ws_bytes = lib.dlb_moe_align_ws_bytes(numel, E)
     ws = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.int32, device=dev)
-    st = lib.dlb_moe_align_block_size(ids.data_ptr(), numel, E, block, s0.data_ptr(), cap,
+    st = lib.dlb_moe_align_block_size(ids.data_ptr(), 0, numel, E, block, s0.data_ptr(), cap,
                                       e0.data_ptr(), nblk, c0.data_ptr(), n0.data_ptr(),
                                       ws.data_ptr(), ws.numel() * 4, stream)
     assert st == 0
     _, _, s1, e1, c1, n1 = _buffers(numel, E, block, dev)
 
     def call_static():
-        st = lib.dlb_moe_align_block_size_static(ids.data_ptr(), numel, E, block, s1.data_ptr(), cap,
+        st = lib.dlb_moe_align_block_size_static(ids.data_ptr(), 0, numel, E, block, s1.data_ptr(), cap,
                                                  e1.data_ptr(), nblk, c1.data_ptr(), n1.data_ptr(),
                                                  stream)
         assert st == 0
@@ -82,7 +82,7 @@ def test_static_scratch_rejects_oversized_input(dev):
     s = torch.empty((cap,), dtype=torch.int32, device=dev)
     e = torch.empty((nblk,), dtype=torch.int32, device=dev)
     n = torch.empty((1,), dtype=torch.int32, device=dev)
-    st = lib.dlb_moe_align_block_size_static(ids.data_ptr(), numel, E, block, s.data_ptr(), cap,
+    st = lib.dlb_moe_align_block_size_static(ids.data_ptr(), 0, numel, E, block, s.data_ptr(), cap,
                                              e.data_ptr(), nblk, None, n.data_ptr(),
                                              _lib.current_stream_ptr(dev))
     assert st == -4  # DLB_ERR_WORKSPACE
